@@ -2,6 +2,10 @@
 
 from .plan import (  # noqa: F401
     AttentionSpec,
+    CausalConvSpec,
+    GateSpec,
+    LatentAttentionSpec,
+    RoutedFFNSpec,
     DenseFFNSpec,
     HeadSpec,
     LayerSpec,
@@ -21,3 +25,4 @@ from .registry import (  # noqa: F401
     supported_architectures,
 )
 from .gpt2 import GPT2Config  # noqa: F401  (registers itself)
+from .bokulix import BokulixConfig  # noqa: F401  (registers itself)

@@ -47,7 +47,7 @@ class TensorSource:
 
 @dataclass(frozen=True)
 class NormSpec:
-    kind: str  # "layernorm"
+    kind: str  # "layernorm" | "rmsnorm" (weight only)
     width: int
     eps: float
     tensors: dict = field(default_factory=dict)  # "weight", "bias"
@@ -100,10 +100,67 @@ class DenseFFNSpec:
 
 
 @dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Attention over one compressed row a position: the row c (`rank` wide, normalised) is what the cache
+    keeps, and each head's keys (`head_dim` wide) and values (`value_dim` wide) are linear in it. No
+    position enters the scores. `window` as in AttentionSpec; `gated`: the heads' outputs are
+    multiplied by the sigmoid of a projection of the mixer's input before the output projection."""
+
+    kind: str  # "latent_attention"
+    width: int
+    n_head: int
+    head_dim: int
+    value_dim: int
+    rank: int
+    scale: float
+    window: int  # 0 = every earlier position
+    eps: float  # of the compressed row's norm
+    gated: bool = True
+    tensors: dict = field(default_factory=dict)  # q, down, down_norm, up_k, up_v, gate, out
+
+
+@dataclass(frozen=True)
+class RoutedFFNSpec:
+    """A mixture of gated feed-forward units: each token takes the `top` experts with the largest router
+    logits, weighted by the softmax over those logits alone. Expert: down(act(gate h) * (up h))."""
+
+    kind: str  # "routed_ffn"
+    width: int
+    inner: int
+    n_experts: int
+    top: int
+    activation: str  # "silu"
+    tensors: dict = field(default_factory=dict)  # router, router_bias, and per expert e: ("gate", e), ("up", e), ("down", e)
+
+
+@dataclass(frozen=True)
+class CausalConvSpec:
+    """A causal convolution over time on each channel of what a sublayer reads: h <- h + conv(h),
+    `taps` inputs back; the last taps - 1 inputs are part of a request's state."""
+
+    kind: str  # "causal_conv"
+    width: int
+    taps: int
+    tensors: dict = field(default_factory=dict)  # "weight" [width, taps]
+
+
+@dataclass(frozen=True)
+class GateSpec:
+    """A gate on a sublayer's result: result * sigmoid(W h + b), h the sublayer's input."""
+
+    kind: str  # "sigmoid_gate"
+    width: int
+    tensors: dict = field(default_factory=dict)  # "weight" [width, width], "bias"
+
+
+@dataclass(frozen=True)
 class LayerSpec:
     """One block: which parts it has and how they are arranged.
 
     arrangement "pre_norm": x += mixer(norm_mixer(x)); x += ffn(norm_ffn(x)).
+    arrangement "post_norm_gated": x += norm_mixer(gate_mixer * mixer(conv(x))); x += norm_ffn(gate_ffn *
+    ffn(x)): the sublayers read the stream itself, the norms stand on their results; `input_conv`
+    (what the mixer reads is first convolved over time) and the gates are optional.
     """
 
     mixer: Any
@@ -111,6 +168,9 @@ class LayerSpec:
     norm_mixer: Any
     norm_ffn: Any
     arrangement: str = "pre_norm"
+    input_conv: Any = None
+    gate_mixer: Any = None
+    gate_ffn: Any = None
 
 
 @dataclass(frozen=True)

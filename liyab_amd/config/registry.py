@@ -44,6 +44,9 @@ def architecture_name_of(raw: dict) -> str:
     archs = raw.get("architectures")
     if isinstance(archs, list) and archs and isinstance(archs[0], str):
         return archs[0]
+    arch = raw.get("architecture")
+    if isinstance(arch, str):
+        return arch
     mt = raw.get("model_type")
     if isinstance(mt, str):
         if mt in _MODEL_TYPES:
@@ -51,7 +54,7 @@ def architecture_name_of(raw: dict) -> str:
         raise Unsupported(
             f"architecture '{mt}' is not supported yet (supported: {supported_architectures()})"
         )
-    raise InvalidModel("not a model folder: config.json has neither 'architectures' nor 'model_type'")
+    raise InvalidModel("not a model folder: config.json has neither 'architectures' nor 'architecture' nor 'model_type'")
 
 
 def config_from_dict(raw: dict):

@@ -1,0 +1,262 @@
+// Many small products with one launch: out rows of group g = a rows . w[g]^T, where a group is a
+// head (every row of the step, its own columns of `a` and of `out`) or an expert (the rows that a
+// router sent to it, listed in tiles of kGroupedRows places by liyab_moe_align).
+//
+//   idx   = the row's number: m for heads; rows_list[place] for listed rows (-1: an empty place)
+//   a row = a + (idx / a_div) * lda + g * a_group_cols       (a_div: entries a token, so that a
+//                                                             token's row serves each of its experts)
+//   w[g]  = w + g * N * K, a row an output feature ([N, K], K contiguous)
+//   out   = out + idx * ldo + g * out_group_cols + column
+//   value = acc0                                 (one matrix)
+//         = silu(acc0) * acc1                    (two matrices: a gated unit's first products)
+//     then * row_scale[idx] (a router's weight), * sigmoid(gate[idx * gate_stride + g * N + column])
+//     (the gate's logits float32 or bfloat16)
+//
+// bfloat16 operands with K a multiple of 8 run on the matrix cores in tiles of 64 x 64 (four waves
+// of 32 x 32, K in steps of 64 through LDS, 32-bit sums); float32 operands, and sizes the matrix
+// kernel does not take, run as plain multiply-adds in 32-bit (tiles of 64 x 64, a thread 4 x 4).
+// Every output element is a sum over k in one order whatever rows share its tile.
+#include "common.h"
+#include "launchers.h"
+
+namespace liyab {
+
+constexpr int kGroupedRows = 64;  // rows a tile; liyab_moe_align lays its lists out in these
+
+struct GroupedParams {
+    const void* a;
+    int64_t lda;
+    int a_div, a_group_cols;
+    const void* w0;
+    const void* w1;
+    void* out;
+    int64_t ldo;
+    int out_group_cols, out_dtype;
+    const int* rows_list;   // null: rows 0..M-1 and the group is blockIdx.z
+    const int* tile_group;  // with rows_list: the group of each tile of rows, -1 for a tile nobody uses
+    const float* row_scale;
+    const void* gate;  // logits of a gate on the output, float32 or bfloat16 (gate_dtype), or null
+    int64_t gate_stride;
+    int gate_dtype;
+    int M, N, K;
+};
+
+__device__ __forceinline__ float gp_sigmoid(float z) { return 1.0f / (1.0f + expf(-z)); }
+
+template <int NW>
+__device__ __forceinline__ void grouped_store(const GroupedParams& p, int idx, int g, int n, float v0, float v1) {
+    float v = v0;
+    if constexpr (NW == 2) v = v0 * gp_sigmoid(v0) * v1;
+    if (p.row_scale != nullptr) v *= p.row_scale[idx];
+    if (p.gate != nullptr) {
+        const int64_t ga = static_cast<int64_t>(idx) * p.gate_stride + static_cast<int64_t>(g) * p.N + n;
+        v *= gp_sigmoid(p.gate_dtype == kF32 ? static_cast<const float*>(p.gate)[ga] : bf16_to_float(static_cast<const bf16_t*>(p.gate)[ga]));
+    }
+    const int64_t at = static_cast<int64_t>(idx) * p.ldo + static_cast<int64_t>(g) * p.out_group_cols + n;
+    if (p.out_dtype == kF32)
+        static_cast<float*>(p.out)[at] = v;
+    else
+        static_cast<bf16_t*>(p.out)[at] = float_to_bf16(v);
+}
+
+// The rows of this workgroup's tile: their numbers into `idx` (LDS, kGroupedRows ints), the group returned (-1: nothing to do).
+__device__ __forceinline__ int grouped_rows(const GroupedParams& p, int* idx) {
+    const int tile = blockIdx.x;
+    int g;
+    if (p.rows_list != nullptr) {
+        g = p.tile_group[tile];
+        if (g < 0) return -1;
+        for (int i = threadIdx.x; i < kGroupedRows; i += blockDim.x) idx[i] = p.rows_list[tile * kGroupedRows + i];
+    } else {
+        g = blockIdx.z;
+        for (int i = threadIdx.x; i < kGroupedRows; i += blockDim.x) {
+            const int m = tile * kGroupedRows + i;
+            idx[i] = m < p.M ? m : -1;
+        }
+    }
+    __syncthreads();
+    return g;
+}
+
+typedef __attribute__((ext_vector_type(8))) __bf16 gp_bf16x8;
+typedef __attribute__((ext_vector_type(16))) float gp_floatx16;
+typedef __attribute__((ext_vector_type(4))) uint32_t gp_u32x4;
+
+constexpr int GPK = 64;       // k per LDS tile
+constexpr int GPLD = GPK + 8;  // padded row, in elements
+
+template <int NW>
+__global__ void __launch_bounds__(256)
+grouped_mfma_kernel(GroupedParams p) {
+    __shared__ __attribute__((aligned(16))) bf16_t lds[(1 + NW) * 64 * GPLD];
+    __shared__ int idx[kGroupedRows];
+    const int g = grouped_rows(p, idx);
+    if (g < 0) return;
+    const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+    const int wm = wave / 2, wn = wave % 2;
+    const int n0 = blockIdx.y * 64;
+    const int li = lane % 32, lk = (lane / 32) * 8;
+    const int N = p.N, K = p.K;
+    const bf16_t* a = static_cast<const bf16_t*>(p.a) + static_cast<int64_t>(g) * p.a_group_cols;
+    const bf16_t* w[2] = {static_cast<const bf16_t*>(p.w0) + static_cast<int64_t>(g) * N * K,
+                          NW == 2 ? static_cast<const bf16_t*>(p.w1) + static_cast<int64_t>(g) * N * K : nullptr};
+    gp_floatx16 acc[NW];
+#pragma unroll
+    for (int u = 0; u < NW; ++u)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[u][r] = 0.0f;
+
+    // a thread's two 16-byte pieces of each operand tile: rows tid / 8 and tid / 8 + 32, k piece tid % 8
+    const int row_a = tid / 8, kc = (tid % 8) * 8;
+    const bf16_t* a_src[2];
+    const bf16_t* w_src[NW][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int id = idx[row_a + 32 * i];
+        a_src[i] = id >= 0 ? a + static_cast<int64_t>(id / p.a_div) * p.lda : nullptr;
+        const int n = n0 + row_a + 32 * i;
+#pragma unroll
+        for (int u = 0; u < NW; ++u) w_src[u][i] = n < N ? w[u] + static_cast<int64_t>(n) * K : nullptr;
+    }
+    const gp_u32x4 zero = {0, 0, 0, 0};
+    for (int k0 = 0; k0 < K; k0 += GPK) {
+        gp_u32x4 ra[2], rw[NW][2];
+        const bool in_k = k0 + kc < K;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            ra[i] = (a_src[i] != nullptr && in_k) ? *reinterpret_cast<const gp_u32x4*>(a_src[i] + k0 + kc) : zero;
+#pragma unroll
+            for (int u = 0; u < NW; ++u) rw[u][i] = (w_src[u][i] != nullptr && in_k) ? *reinterpret_cast<const gp_u32x4*>(w_src[u][i] + k0 + kc) : zero;
+        }
+        __syncthreads();  // the previous tile's fragments have been read
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            *reinterpret_cast<gp_u32x4*>(lds + (row_a + 32 * i) * GPLD + kc) = ra[i];
+#pragma unroll
+            for (int u = 0; u < NW; ++u) *reinterpret_cast<gp_u32x4*>(lds + ((1 + u) * 64 + row_a + 32 * i) * GPLD + kc) = rw[u][i];
+        }
+        __syncthreads();
+        const bf16_t* Ab = lds + (wm * 32 + li) * GPLD + lk;
+#pragma unroll
+        for (int ks = 0; ks < GPK; ks += 16) {
+            const gp_bf16x8 fa = *reinterpret_cast<const gp_bf16x8*>(Ab + ks);
+#pragma unroll
+            for (int u = 0; u < NW; ++u) {
+                const gp_bf16x8 fw = *reinterpret_cast<const gp_bf16x8*>(lds + ((1 + u) * 64 + wn * 32 + li) * GPLD + lk + ks);
+                acc[u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fw, acc[u], 0, 0, 0);
+            }
+        }
+    }
+    // C block layout: a lane holds column li; rows 8 * (r / 4) + 4 * (lane / 32) + r % 4
+    const int n = n0 + wn * 32 + li;
+    if (n >= N) return;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int id = idx[wm * 32 + 4 * (lane / 32) + 8 * (r / 4) + r % 4];
+        if (id >= 0) grouped_store<NW>(p, id, g, n, acc[0][r], NW == 2 ? acc[NW - 1][r] : 0.0f);
+    }
+}
+
+// Plain 32-bit multiply-adds: a tile of 64 rows x 64 output features, a thread 4 x 4 of them, K in
+// steps of 16 through LDS. Takes every size and both element types.
+template <typename T, int NW>
+__global__ void __launch_bounds__(256)
+grouped_plain_kernel(GroupedParams p) {
+    constexpr int BK = 16;
+    __shared__ float la[BK][64 + 1];
+    __shared__ float lw[NW][BK][64 + 1];
+    __shared__ int idx[kGroupedRows];
+    const int g = grouped_rows(p, idx);
+    if (g < 0) return;
+    const int tid = threadIdx.x;
+    const int n0 = blockIdx.y * 64;
+    const int N = p.N, K = p.K;
+    const T* a = static_cast<const T*>(p.a) + static_cast<int64_t>(g) * p.a_group_cols;
+    const T* w[2] = {static_cast<const T*>(p.w0) + static_cast<int64_t>(g) * N * K,
+                     NW == 2 ? static_cast<const T*>(p.w1) + static_cast<int64_t>(g) * N * K : nullptr};
+    const int tr = (tid / 16) * 4, tc = (tid % 16) * 4;  // this thread's rows and columns of the tile
+    float acc[NW][4][4];
+#pragma unroll
+    for (int u = 0; u < NW; ++u)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[u][i][j] = 0.0f;
+    for (int k0 = 0; k0 < K; k0 += BK) {
+        __syncthreads();
+        // 64 x 16 values of each operand: a thread four of them, k fastest
+        for (int e = tid; e < 64 * BK; e += 256) {
+            const int row = e / BK, k = k0 + e % BK;
+            const int id = idx[row];
+            la[e % BK][row] = (id >= 0 && k < K) ? to_float<T>(a[static_cast<int64_t>(id / p.a_div) * p.lda + k]) : 0.0f;
+            const int n = n0 + row;
+#pragma unroll
+            for (int u = 0; u < NW; ++u) lw[u][e % BK][row] = (n < N && k < K) ? to_float<T>(w[u][static_cast<int64_t>(n) * K + k]) : 0.0f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < BK; ++k) {
+            float av[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) av[i] = la[k][tr + i];
+#pragma unroll
+            for (int u = 0; u < NW; ++u) {
+                float wv[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) wv[j] = lw[u][k][tc + j];
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) acc[u][i][j] = fmaf(av[i], wv[j], acc[u][i][j]);
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int id = idx[tr + i];
+        if (id < 0) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int n = n0 + tc + j;
+            if (n < N) grouped_store<NW>(p, id, g, n, acc[0][i][j], NW == 2 ? acc[NW - 1][i][j] : 0.0f);
+        }
+    }
+}
+
+}  // namespace liyab
+
+using namespace liyab;
+
+// See the head of this file. dtype: the element type of a, w0 and w1. n_groups: heads (rows_list
+// null) or experts (the values of tile_group lie below it; the caller has made them so). n_tiles:
+// the tiles of rows to launch (with rows_list: the length of tile_group; without: (M + 63) / 64).
+extern "C" int liyab_grouped_product(const void* a, int64_t lda, int a_div, int a_group_cols, const void* w0, const void* w1, int dtype,
+                                     void* out, int out_dtype, int64_t ldo, int out_group_cols, const int* rows_list,
+                                     const int* tile_group, int n_tiles, int n_groups, const float* row_scale, const void* gate,
+                                     int gate_dtype, int64_t gate_stride, int M, int N, int K, hipStream_t stream) {
+    LIYAB_REQUIRE(a && w0 && out, "grouped_product: null pointer");
+    LIYAB_REQUIRE(dtype == kF32 || dtype == kBF16, "grouped_product: unknown dtype %d", dtype);
+    LIYAB_REQUIRE(out_dtype == kF32 || out_dtype == kBF16, "grouped_product: unknown output dtype %d", out_dtype);
+    LIYAB_REQUIRE(M >= 0 && N > 0 && K > 0 && a_div >= 1 && n_groups >= 1 && n_groups <= 65535 && n_tiles >= 0, "grouped_product: bad sizes M=%d N=%d K=%d", M, N, K);
+    LIYAB_REQUIRE((rows_list == nullptr) == (tile_group == nullptr), "grouped_product: a list of rows goes with the groups of its tiles");
+    LIYAB_REQUIRE(rows_list != nullptr || n_tiles == (M + kGroupedRows - 1) / kGroupedRows, "grouped_product: %d tiles for %d rows", n_tiles, M);
+    LIYAB_REQUIRE(gate == nullptr || gate_dtype == kF32 || gate_dtype == kBF16, "grouped_product: unknown gate dtype %d", gate_dtype);
+    LIYAB_REQUIRE(gate == nullptr || gate_stride >= static_cast<int64_t>(rows_list ? 1 : n_groups) * N, "grouped_product: the gate's rows are shorter than the output's");
+    if (M == 0 || n_tiles == 0) return 0;
+    GroupedParams p{a, lda, a_div, a_group_cols, w0, w1, out, ldo, out_group_cols, out_dtype, rows_list, tile_group, row_scale, gate, gate_stride, gate_dtype, M, N, K};
+    const dim3 grid(n_tiles, (N + 63) / 64, rows_list ? 1 : n_groups);
+    const bool matrix = dtype == kBF16 && K % 8 == 0 && lda % 8 == 0 && a_group_cols % 8 == 0 &&
+                        (reinterpret_cast<uintptr_t>(a) & 15) == 0 && (reinterpret_cast<uintptr_t>(w0) & 15) == 0 &&
+                        (reinterpret_cast<uintptr_t>(w1) & 15) == 0;
+    if (matrix) {
+        if (w1 != nullptr) grouped_mfma_kernel<2><<<grid, 256, 0, stream>>>(p);
+        else grouped_mfma_kernel<1><<<grid, 256, 0, stream>>>(p);
+    } else if (dtype == kBF16) {
+        if (w1 != nullptr) grouped_plain_kernel<bf16_t, 2><<<grid, 256, 0, stream>>>(p);
+        else grouped_plain_kernel<bf16_t, 1><<<grid, 256, 0, stream>>>(p);
+    } else {
+        if (w1 != nullptr) grouped_plain_kernel<float, 2><<<grid, 256, 0, stream>>>(p);
+        else grouped_plain_kernel<float, 1><<<grid, 256, 0, stream>>>(p);
+    }
+    return check_launch("grouped_product");
+}

@@ -57,4 +57,24 @@ int liyab_attention_prefill(void* out, int64_t out_stride, const void* q, int64_
                             const int* block_tables, int max_blocks, const int* work, int n_tiles, int tile, int ksplit, float scale,
                             int window, int n_head, int n_kv_head, int hd, int page_size, int num_pages, hipStream_t stream);
 
+int liyab_rmsnorm(void* out, int out_dtype, const float* x, const float* w, const int* rows, int n, int d, float eps, hipStream_t stream);
+int liyab_gated_norm_add(float* x, void* cast_out, int cast_dtype, const float* y, int n_sum, const float* gate, int64_t gate_stride,
+                         const float* w, float eps, int normalize, int n, int d, float* state, int ring, int n_slots,
+                         const int* tok_seq, const int* positions, const int* context_lens, const int* state_slots, const int* n_real,
+                         hipStream_t stream);
+int liyab_causal_conv(void* out, void* cast_out, int dtype, const float* x, const float* w, int taps, const float* state, int n_slots,
+                      const int* tok_seq, const int* positions, const int* seq_starts, const int* state_slots, int n, int d,
+                      hipStream_t stream);
+int liyab_keep_rows(float* state, int ring, int n_slots, const float* x, const int* tok_seq, const int* positions,
+                    const int* context_lens, const int* state_slots, const int* n_real, int n, int d, hipStream_t stream);
+int liyab_latent_store(void* cache, int dtype, const void* src, int64_t src_stride, int col_off, const float* w, float eps,
+                       const int* slots, int n, int rank, int page_size, int num_pages, hipStream_t stream);
+int liyab_grouped_product(const void* a, int64_t lda, int a_div, int a_group_cols, const void* w0, const void* w1, int dtype, void* out,
+                          int out_dtype, int64_t ldo, int out_group_cols, const int* rows_list, const int* tile_group, int n_tiles,
+                          int n_groups, const float* row_scale, const void* gate, int gate_dtype, int64_t gate_stride, int M, int N,
+                          int K, hipStream_t stream);
+int liyab_moe_route(const float* logits, int64_t ld, int n, int n_experts, int top, int* ids, float* weights, hipStream_t stream);
+int liyab_moe_align(const int* ids, int n_entries, int n_experts, int block, int* rows_list, int* tile_group, int max_tiles,
+                    hipStream_t stream);
+
 }  // extern "C"

@@ -1,0 +1,113 @@
+// Routing of a mixture of experts: who goes where, before the experts' products run
+// (grouped_product.hip).
+//
+// liyab_moe_route: from each token's 32-bit router logits the `top` experts with the largest
+// logits (among equal logits the lower number first) and their weights, the softmax over the chosen
+// logits alone, in 32-bit. ids and weights [n, top]: entry t * top + k is token t's k-th choice.
+//
+// liyab_moe_align: the entries listed by expert, each expert's stretch padded to whole tiles of
+// `block` places: rows_list [max_tiles * block] (an entry's number, -1 for an empty place) and
+// tile_group [max_tiles] (the expert of each tile, -1 for a tile that is not used). max_tiles is
+// a bound that the step's sizes fix (entries / block + min(experts, entries), rounded up), so
+// that the products' grids do not depend on where the tokens went. One workgroup.
+#include "common.h"
+#include "launchers.h"
+
+namespace liyab {
+
+constexpr int kMaxTop = 32;
+
+__global__ void __launch_bounds__(256)
+moe_route_kernel(const float* __restrict__ logits, int64_t ld, int n, int E, int top, int* __restrict__ ids, float* __restrict__ weights) {
+    const int t = blockIdx.x * 256 + threadIdx.x;
+    if (t >= n) return;
+    const float* z = logits + static_cast<int64_t>(t) * ld;
+    int chosen[kMaxTop];
+    float value[kMaxTop];
+    for (int k = 0; k < top; ++k) {
+        int best = -1;
+        float bv = 0.0f;
+        for (int e = 0; e < E; ++e) {
+            bool taken = false;
+            for (int j = 0; j < k; ++j) taken = taken || chosen[j] == e;
+            const float v = z[e];
+            if (!taken && (best < 0 || v > bv)) {
+                best = e;
+                bv = v;
+            }
+        }
+        chosen[k] = best;
+        value[k] = bv;
+    }
+    float sum = 0.0f;
+    const float largest = value[0];  // the first choice holds the largest logit
+    for (int k = 0; k < top; ++k) {
+        value[k] = expf(value[k] - largest);
+        sum += value[k];
+    }
+    for (int k = 0; k < top; ++k) {
+        ids[static_cast<int64_t>(t) * top + k] = chosen[k];
+        weights[static_cast<int64_t>(t) * top + k] = value[k] / sum;
+    }
+}
+
+__global__ void __launch_bounds__(1024)
+moe_align_kernel(const int* __restrict__ ids, int n_entries, int E, int block, int* __restrict__ rows_list, int* __restrict__ tile_group,
+                 int max_tiles) {
+    extern __shared__ int sh[];  // counts [E], first place of each expert [E + 1]
+    int* counts = sh;
+    int* first = sh + E;
+    const int tid = threadIdx.x;
+    for (int e = tid; e < E; e += 1024) counts[e] = 0;
+    for (int i = tid; i < max_tiles * block; i += 1024) rows_list[i] = -1;
+    for (int i = tid; i < max_tiles; i += 1024) tile_group[i] = -1;
+    __syncthreads();
+    for (int i = tid; i < n_entries; i += 1024) {
+        const int e = ids[i];
+        if (e >= 0 && e < E) atomicAdd(&counts[e], 1);
+    }
+    __syncthreads();
+    if (tid == 0) {
+        int at = 0;
+        for (int e = 0; e < E; ++e) {
+            first[e] = at;
+            const int tiles = (counts[e] + block - 1) / block;
+            for (int i = 0; i < tiles; ++i)
+                if (at / block + i < max_tiles) tile_group[at / block + i] = e;
+            at += tiles * block;
+            counts[e] = 0;  // counts the entries placed so far from here on
+        }
+        first[E] = at;
+    }
+    __syncthreads();
+    for (int i = tid; i < n_entries; i += 1024) {
+        const int e = ids[i];
+        if (e < 0 || e >= E) continue;
+        const int place = first[e] + atomicAdd(&counts[e], 1);
+        if (place < max_tiles * block) rows_list[place] = i;
+    }
+}
+
+}  // namespace liyab
+
+using namespace liyab;
+
+extern "C" int liyab_moe_route(const float* logits, int64_t ld, int n, int n_experts, int top, int* ids, float* weights, hipStream_t stream) {
+    LIYAB_REQUIRE(logits && ids && weights, "moe_route: null pointer");
+    LIYAB_REQUIRE(n >= 0 && n_experts > 0 && top >= 1 && top <= n_experts && top <= kMaxTop && ld >= n_experts,
+                  "moe_route: bad sizes n=%d experts=%d top=%d (at most %d choices a token)", n, n_experts, top, kMaxTop);
+    if (n == 0) return 0;
+    moe_route_kernel<<<(n + 255) / 256, 256, 0, stream>>>(logits, ld, n, n_experts, top, ids, weights);
+    return check_launch("moe_route");
+}
+
+extern "C" int liyab_moe_align(const int* ids, int n_entries, int n_experts, int block, int* rows_list, int* tile_group, int max_tiles,
+                               hipStream_t stream) {
+    LIYAB_REQUIRE(ids && rows_list && tile_group, "moe_align: null pointer");
+    LIYAB_REQUIRE(n_entries >= 0 && n_experts > 0 && n_experts <= 4096 && block > 0, "moe_align: bad sizes (at most 4,096 experts)");
+    LIYAB_REQUIRE(static_cast<int64_t>(max_tiles) * block >= static_cast<int64_t>(n_entries) + static_cast<int64_t>(n_entries < n_experts ? n_entries : n_experts) * (block - 1),
+                  "moe_align: %d tiles of %d places do not hold %d entries of %d experts", max_tiles, block, n_entries, n_experts);
+    if (n_entries == 0) return 0;
+    moe_align_kernel<<<1, 1024, (2 * n_experts + 1) * sizeof(int), stream>>>(ids, n_entries, n_experts, block, rows_list, tile_group, max_tiles);
+    return check_launch("moe_align");
+}

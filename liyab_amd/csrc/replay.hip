@@ -87,6 +87,14 @@ static const Entry kEntries[] = {
     LIYAB_ENTRY(liyab_attention_decode),
     LIYAB_ENTRY(liyab_attention_merge),
     LIYAB_ENTRY(liyab_attention_prefill),
+    LIYAB_ENTRY(liyab_rmsnorm),
+    LIYAB_ENTRY(liyab_gated_norm_add),
+    LIYAB_ENTRY(liyab_causal_conv),
+    LIYAB_ENTRY(liyab_keep_rows),
+    LIYAB_ENTRY(liyab_latent_store),
+    LIYAB_ENTRY(liyab_grouped_product),
+    LIYAB_ENTRY(liyab_moe_route),
+    LIYAB_ENTRY(liyab_moe_align),
 };
 constexpr int kNumEntries = static_cast<int>(sizeof(kEntries) / sizeof(kEntries[0]));
 

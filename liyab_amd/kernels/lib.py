@@ -72,6 +72,15 @@ _SIGNATURES = {
     "liyab_argmax_static_init": [],
     "liyab_argmax_static": [P, P, c_int64, c_int, c_int, P, P, P],
     "liyab_sample": [P, P, c_int64, c_int, c_int, P, P, P, P, P, P, P],
+    "liyab_rmsnorm": [P, c_int, P, P, P, c_int, c_int, c_float, P],
+    "liyab_gated_norm_add": [P, P, c_int, P, c_int, P, c_int64, P, c_float, c_int, c_int, c_int, P, c_int, c_int, P, P, P, P, P, P],
+    "liyab_causal_conv": [P, P, c_int, P, P, c_int, P, c_int, P, P, P, P, c_int, c_int, P],
+    "liyab_keep_rows": [P, c_int, c_int, P, P, P, P, P, P, c_int, c_int, P],
+    "liyab_latent_store": [P, c_int, P, c_int64, c_int, P, c_float, P, c_int, c_int, c_int, c_int, P],
+    "liyab_grouped_product": [P, c_int64, c_int, c_int, P, P, c_int, P, c_int, c_int64, c_int, P, P, c_int, c_int, P, P, c_int, c_int64,
+                              c_int, c_int, c_int, P],
+    "liyab_moe_route": [P, c_int64, c_int, c_int, c_int, P, P, P],
+    "liyab_moe_align": [P, c_int, c_int, c_int, P, P, c_int, P],
 }
 
 

@@ -993,3 +993,227 @@ def attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache
         return
     attention_generic(out, q, k_cache, v_cache, block_tables, ctx.tok_seq, ctx.positions, n_head=n_head, scale=scale,
                       window=window)
+
+
+# -- root-mean-square norms, the gated residual update, the input convolution --------------------
+def rmsnorm(out: torch.Tensor, x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, rows: Optional[torch.Tensor] = None) -> None:
+    """out[r] = x[rows[r]] (or x[r]) / sqrt(mean(.^2) + eps) * weight; x float32 [*, d], out [n, d]
+    float32 or bfloat16."""
+    _dev(out, "out")
+    _dev(x, "x")
+    n, d = out.shape
+    if x.dtype != torch.float32 or x.dim() != 2 or x.shape[1] != d or not x.is_contiguous() or not out.is_contiguous():
+        raise KernelError(f"rmsnorm: x must be contiguous float32 [*, {d}] and out contiguous, got {tuple(x.shape)} {x.dtype}")
+    _f32vec(weight, "norm weight", d)
+    if rows is not None:
+        _i32(rows, "rows", n)
+    elif x.shape[0] < n:
+        raise KernelError("rmsnorm: fewer input rows than output rows")
+    _lib.call("liyab_rmsnorm", out.data_ptr(), dtype_code(out.dtype), x.data_ptr(), _ptr(weight), _ptr(rows), n, d, float(eps), _stream())
+
+
+def _keep_args(keep, d: int):
+    """The arguments that say which rows of a step are kept as a convolution's input history: keep =
+    (state float32 [slots, ring, d], ctx) or None."""
+    if keep is None:
+        return (None, 0, 0, None, None, None, None, None)
+    state, ctx = keep
+    _dev(state, "state")
+    if state.dtype != torch.float32 or state.dim() != 3 or state.shape[2] != d or state.shape[1] < 1 or not state.is_contiguous():
+        raise KernelError(f"kept rows: the state must be contiguous float32 [slots, ring, {d}], got {tuple(state.shape)} {state.dtype}")
+    n = ctx.n_tokens
+    _i32(ctx.tok_seq, "tok_seq", n)
+    _i32(ctx.positions, "positions", n)
+    _i32(ctx.context_lens, "context_lens", ctx.n_seqs)
+    _i32(ctx.state_slots, "state_slots", ctx.n_seqs)
+    _i32(ctx.seq_starts, "seq_starts", ctx.n_seqs + 1)
+    return (state.data_ptr(), state.shape[1], state.shape[0], ctx.tok_seq.data_ptr(), ctx.positions.data_ptr(),
+            ctx.context_lens.data_ptr(), ctx.state_slots.data_ptr(), ctx.seq_starts.data_ptr() + 4 * ctx.n_seqs)
+
+
+def gated_norm_add(x: torch.Tensor, y: torch.Tensor, weight: Optional[torch.Tensor], eps: float, *, n_sum: int = 1,
+                   gate: Optional[torch.Tensor] = None, cast_out: Optional[torch.Tensor] = None, keep=None,
+                   normalize: bool = True) -> None:
+    """x[t] += weight * s / sqrt(mean(s^2) + eps) with s = (y[t * n_sum] + ... + y[t * n_sum + n_sum - 1]) *
+    sigmoid(gate[t]); x float32 [n, d] in place, y float32 [n * n_sum, d], gate float32 [n, d] (rows may
+    be strided: columns of a wider product) or None. `cast_out` [n, d] (float32 or bfloat16) gets the new
+    rows rounded. `keep` = (state, ctx): before the update, the last rows of each request go to its input
+    history, state[slot, position % ring] (the rows behind the step's tokens are left out). Without
+    `normalize`: x[t] += s."""
+    _dev(x, "x")
+    _dev(y, "y")
+    n, d = x.shape
+    if x.dtype != torch.float32 or not x.is_contiguous():
+        raise KernelError("gated_norm_add: x must be contiguous float32 [n, d]")
+    if y.dtype != torch.float32 or not y.is_contiguous() or y.numel() != n * n_sum * d or n_sum < 1:
+        raise KernelError(f"gated_norm_add: y must be contiguous float32 with {n_sum} rows of {d} a token, got {tuple(y.shape)} {y.dtype}")
+    _f32vec(weight, "norm weight", d)
+    gs = 0
+    if gate is not None:
+        gs = _rows(gate, "gate")
+        if gate.dtype != torch.float32 or tuple(gate.shape) != (n, d):
+            raise KernelError(f"gated_norm_add: the gate must be float32 [{n}, {d}], got {tuple(gate.shape)} {gate.dtype}")
+    code = F32
+    if cast_out is not None:
+        _dev(cast_out, "cast_out")
+        if tuple(cast_out.shape) != (n, d) or not cast_out.is_contiguous():
+            raise KernelError(f"gated_norm_add: cast_out must be contiguous [{n}, {d}]")
+        code = dtype_code(cast_out.dtype)
+    if keep is not None and keep[1].n_tokens != n:
+        raise KernelError("gated_norm_add: rows are kept for a step of as many rows as x has")
+    _lib.call("liyab_gated_norm_add", x.data_ptr(), _ptr(cast_out), code, y.data_ptr(), n_sum, _ptr(gate), gs, _ptr(weight), float(eps),
+              1 if normalize else 0, n, d, *_keep_args(keep, d), _stream())
+
+
+def keep_rows(x: torch.Tensor, state: torch.Tensor, ctx) -> None:
+    """The last rows of each request in the step go to its input history (see `gated_norm_add`'s `keep`)."""
+    _dev(x, "x")
+    n, d = x.shape
+    if x.dtype != torch.float32 or not x.is_contiguous() or ctx.n_tokens != n:
+        raise KernelError("keep_rows: x must be the step's contiguous float32 rows")
+    a = _keep_args((state, ctx), d)
+    _lib.call("liyab_keep_rows", a[0], a[1], a[2], x.data_ptr(), *a[3:], n, d, _stream())
+
+
+CONV_MAX_TAPS = 16
+
+
+def causal_conv(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, state: Optional[torch.Tensor], ctx,
+                cast_out: Optional[torch.Tensor] = None) -> None:
+    """out[t] = x[t] + sum_j weight[:, j] * x[t - taps + 1 + j] over each request's own tokens in time, zeros
+    before its start; x float32 [n, d] (the step's rows), weight float32 [d, taps], state float32 [slots,
+    taps - 1, d] (position p of a request at ring place p % (taps - 1)) for what lies before the step's
+    portion. out (and cast_out = x rounded) [n, d] float32 or bfloat16."""
+    _dev(out, "out")
+    _dev(x, "x")
+    n, d = x.shape
+    if x.dtype != torch.float32 or not x.is_contiguous() or ctx.n_tokens != n:
+        raise KernelError("causal_conv: x must be the step's contiguous float32 rows")
+    if tuple(out.shape) != (n, d) or not out.is_contiguous():
+        raise KernelError(f"causal_conv: out must be contiguous [{n}, {d}]")
+    if cast_out is not None and (tuple(cast_out.shape) != (n, d) or not cast_out.is_contiguous() or cast_out.dtype != out.dtype):
+        raise KernelError("causal_conv: cast_out must match out")
+    _dev(weight, "weight")
+    if weight.dtype != torch.float32 or weight.dim() != 2 or weight.shape[0] != d or not weight.is_contiguous():
+        raise KernelError(f"causal_conv: the weight must be contiguous float32 [{d}, taps], got {tuple(weight.shape)} {weight.dtype}")
+    taps = weight.shape[1]
+    if not 1 <= taps <= CONV_MAX_TAPS:
+        raise KernelError(f"causal_conv: {taps} taps; 1 to {CONV_MAX_TAPS} are taken")
+    n_slots = 0
+    if taps > 1:
+        if state is None or state.dtype != torch.float32 or tuple(state.shape[1:]) != (taps - 1, d) or not state.is_contiguous():
+            raise KernelError(f"causal_conv: the state must be contiguous float32 [slots, {taps - 1}, {d}]")
+        _dev(state, "state")
+        n_slots = state.shape[0]
+    _i32(ctx.tok_seq, "tok_seq", n)
+    _i32(ctx.positions, "positions", n)
+    _i32(ctx.seq_starts, "seq_starts", ctx.n_seqs + 1)
+    _i32(ctx.state_slots, "state_slots", ctx.n_seqs)
+    _lib.call("liyab_causal_conv", out.data_ptr(), _ptr(cast_out), dtype_code(out.dtype), x.data_ptr(), weight.data_ptr(), taps,
+              _ptr(state) if taps > 1 else None, n_slots, ctx.tok_seq.data_ptr(), ctx.positions.data_ptr(), ctx.seq_starts.data_ptr(),
+              ctx.state_slots.data_ptr(), n, d, _stream())
+
+
+# -- latent attention's cached row, products a head, routed experts -------------------------------
+def latent_store(cache: torch.Tensor, src: torch.Tensor, col_off: int, weight: Optional[torch.Tensor], eps: float,
+                 slots: torch.Tensor, num_pages: Optional[int] = None) -> None:
+    """cache[slot of t] = rmsnorm(src[t, col_off : col_off + rank]) * weight for each row t of the step; cache
+    [pages, 1, page_size, rank] in src's dtype; slots int32 [n] = page * page_size + offset (a slot outside
+    the pages is not written)."""
+    _dev(cache, "cache")
+    if cache.dim() != 4 or cache.shape[1] != 1 or not cache.is_contiguous() or cache.dtype != src.dtype:
+        raise KernelError(f"latent_store: the cache must be contiguous [pages, 1, page_size, rank] in the rows' dtype, got {tuple(cache.shape)}")
+    stride = _rows(src, "src")
+    n, rank = src.shape[0], cache.shape[3]
+    if col_off < 0 or col_off + rank > src.shape[1]:
+        raise KernelError("latent_store: the columns pass the source's width")
+    _f32vec(weight, "norm weight", rank)
+    _i32(slots, "slots", n)
+    _lib.call("liyab_latent_store", cache.data_ptr(), dtype_code(src.dtype), src.data_ptr(), stride, col_off, _ptr(weight), float(eps),
+              slots.data_ptr(), n, rank, cache.shape[2], _pages(cache, num_pages), _stream())
+
+
+GROUPED_ROWS = 64  # rows a tile of the grouped product (csrc/grouped_product.hip: kGroupedRows)
+
+
+def heads_product(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, gate: Optional[torch.Tensor] = None) -> None:
+    """out[t, h * N + j] = sum_k a[t, h * K + k] * w[h, j, k] (* sigmoid(gate[t, h * N + j])): a product of
+    its own for every head. a [n, >= H * K] and out [n, >= H * N] may be column ranges of wider rows; w
+    [H, N, K] contiguous in a's dtype; gate float32 or bfloat16 logits, or None."""
+    _dev(w, "w")
+    if w.dim() != 3 or not w.is_contiguous() or w.dtype != a.dtype:
+        raise KernelError(f"heads_product: w must be contiguous [heads, N, K] in a's dtype, got {tuple(w.shape)} {w.dtype}")
+    H, N, K = w.shape
+    lda, ldo = _rows(a, "a"), _rows(out, "out")
+    n = a.shape[0]
+    if a.shape[1] != H * K or tuple(out.shape) != (n, H * N):
+        raise KernelError(f"heads_product: a {tuple(a.shape)} / out {tuple(out.shape)} do not fit {H} heads of {K} -> {N}")
+    gs = 0
+    if gate is not None:
+        gs = _rows(gate, "gate")
+        if tuple(gate.shape) != (n, H * N):
+            raise KernelError(f"heads_product: the gate must be [{n}, {H * N}]")
+    _lib.call("liyab_grouped_product", a.data_ptr(), lda, 1, K, w.data_ptr(), None, dtype_code(a.dtype), out.data_ptr(),
+              dtype_code(out.dtype), ldo, N, None, None, (n + GROUPED_ROWS - 1) // GROUPED_ROWS, H, None, _ptr(gate),
+              dtype_code(gate.dtype) if gate is not None else F32, gs, n, N, K, _stream())
+
+
+MOE_MAX_TOP = 32
+
+
+def moe_tiles(n_entries: int, n_experts: int) -> int:
+    """The tiles of GROUPED_ROWS places that hold `n_entries` entries listed by expert, whatever their
+    experts: a bound that follows from the sizes alone."""
+    return -(-(n_entries + min(n_entries, n_experts) * (GROUPED_ROWS - 1)) // GROUPED_ROWS)
+
+
+def moe_route(logits: torch.Tensor, top: int, ids: torch.Tensor, weights: torch.Tensor, rows_list: torch.Tensor,
+              tile_group: torch.Tensor) -> None:
+    """From float32 router logits [n, experts] (rows may be strided): ids int32 and weights float32 [n,
+    top] (the experts with the largest logits, softmax over those alone), and the entries t * top + k
+    listed by expert in tiles: rows_list int32 [tiles * GROUPED_ROWS] (-1: empty), tile_group int32
+    [tiles] (-1: unused), tiles = moe_tiles(n * top, experts)."""
+    ld = _rows(logits, "logits")
+    n, E = logits.shape
+    if logits.dtype != torch.float32:
+        raise KernelError("moe_route: the logits must be float32")
+    if not 1 <= top <= min(E, MOE_MAX_TOP):
+        raise KernelError(f"moe_route: {top} of {E} experts a token (at most {MOE_MAX_TOP})")
+    tiles = moe_tiles(n * top, E)
+    _i32(ids, "ids", n * top)
+    _i32(rows_list, "rows_list", tiles * GROUPED_ROWS)
+    _i32(tile_group, "tile_group", tiles)
+    _dev(weights, "weights")
+    if weights.dtype != torch.float32 or weights.numel() < n * top or not weights.is_contiguous():
+        raise KernelError("moe_route: weights must be contiguous float32 [n, top]")
+    _lib.call("liyab_moe_route", logits.data_ptr(), ld, n, E, top, ids.data_ptr(), weights.data_ptr(), _stream())
+    _lib.call("liyab_moe_align", ids.data_ptr(), n * top, E, GROUPED_ROWS, rows_list.data_ptr(), tile_group.data_ptr(), tiles, _stream())
+
+
+def moe_product(out: torch.Tensor, a: torch.Tensor, w0: torch.Tensor, w1: Optional[torch.Tensor], rows_list: torch.Tensor,
+                tile_group: torch.Tensor, *, a_div: int = 1, row_scale: Optional[torch.Tensor] = None) -> None:
+    """For every listed entry e of expert g: out[e] = f(a[e // a_div] . w0[g]^T, a[e // a_div] . w1[g]^T) *
+    row_scale[e], f(u, v) = silu(u) * v with two matrices and u with one. a [*, K] and out [entries, N]
+    contiguous, w0 / w1 [experts, N, K] in a's dtype; rows_list and tile_group as `moe_route` leaves them."""
+    _dev(w0, "w0")
+    if w0.dim() != 3 or not w0.is_contiguous() or w0.dtype != a.dtype:
+        raise KernelError(f"moe_product: w0 must be contiguous [experts, N, K] in a's dtype, got {tuple(w0.shape)} {w0.dtype}")
+    E, N, K = w0.shape
+    if w1 is not None and (tuple(w1.shape) != (E, N, K) or not w1.is_contiguous() or w1.dtype != a.dtype):
+        raise KernelError("moe_product: w1 must match w0")
+    lda, ldo = _rows(a, "a"), _rows(out, "out")
+    entries = out.shape[0]
+    if a.shape[1] != K or out.shape[1] != N or a_div < 1 or a.shape[0] * a_div < entries:
+        raise KernelError(f"moe_product: a {tuple(a.shape)} / out {tuple(out.shape)} do not fit [{E}, {N}, {K}] with {a_div} entries a row")
+    tiles = tile_group.numel()
+    if tiles < moe_tiles(entries, E):
+        raise KernelError(f"moe_product: {tiles} tiles do not hold {entries} entries of {E} experts")
+    _i32(rows_list, "rows_list", tiles * GROUPED_ROWS)
+    _i32(tile_group, "tile_group", tiles)
+    if row_scale is not None:
+        _dev(row_scale, "row_scale")
+        if row_scale.dtype != torch.float32 or row_scale.numel() < entries or not row_scale.is_contiguous():
+            raise KernelError("moe_product: row_scale must be contiguous float32 [entries]")
+    _lib.call("liyab_grouped_product", a.data_ptr(), lda, a_div, 0, w0.data_ptr(), _ptr(w1), dtype_code(a.dtype), out.data_ptr(),
+              dtype_code(out.dtype), ldo, 0, rows_list.data_ptr(), tile_group.data_ptr(), tiles, E, _ptr(row_scale), None, F32, 0,
+              entries, N, K, _stream())

@@ -126,7 +126,14 @@ class DecoderModel:
             ffn = build_part("ffn", spec.ffn, store, dtype) if spec.ffn is not None else None
             norm_mixer = build_part("norm", spec.norm_mixer, store, dtype) if spec.norm_mixer is not None else None
             norm_ffn = build_part("norm", spec.norm_ffn, store, dtype) if spec.norm_ffn is not None else None
-            self.blocks.append(find_part("block", spec.arrangement)(spec, mixer, ffn, norm_mixer, norm_ffn))
+            # what a block may have of its own between the stream and its sublayers (a convolution on a
+            # sublayer's input, gates on the results): built here, handed over by name where the plan has them
+            extras = {}
+            for name, family in (("input_conv", "conv"), ("gate_mixer", "gate"), ("gate_ffn", "gate")):
+                extra = getattr(spec, name, None)
+                if extra is not None:
+                    extras[name] = build_part(family, extra, store, dtype)
+            self.blocks.append(find_part("block", spec.arrangement)(spec, mixer, ffn, norm_mixer, norm_ffn, **extras))
         self.final_norm = build_part("norm", plan.final_norm, store, dtype) if plan.final_norm is not None else None
         self.head = build_part("head", plan.head, store, dtype)
         self.order = list(plan.order)
@@ -156,7 +163,7 @@ class DecoderModel:
         # the head see the wanted rows only.
         every = [self.embedding, self.residual_position]
         for block in self.blocks:
-            every += [block] + [getattr(block, a, None) for a in ("mixer", "ffn", "norm_mixer", "norm_ffn")]
+            every += [block] + [getattr(block, a, None) for a in ("mixer", "ffn", "norm_mixer", "norm_ffn", "conv", "gate_mixer", "gate_ffn")]
         self.takes_padding_rows = all(bool(getattr(part, "takes_padding_rows", False)) for part in every if part is not None)
 
     # -- what the cache manager needs to know ---------------------------------
@@ -174,7 +181,9 @@ class DecoderModel:
     def state_specs(self) -> Dict[int, StateSpec]:
         out = {}
         for layer in sorted({e.cache_layer for e in self.order}):
-            spec = self.blocks[layer].mixer.state_spec()
+            block = self.blocks[layer]
+            # a block that keeps state of its own between steps says so; otherwise the mixer's
+            spec = block.state_spec() if hasattr(block, "state_spec") else block.mixer.state_spec()
             if spec is not None:
                 out[layer] = spec
         return out

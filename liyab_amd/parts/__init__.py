@@ -5,12 +5,14 @@ from .registry import (  # noqa: F401
     build_part,
     find_part,
     register_block,
+    register_conv,
     register_embedding,
     register_ffn,
+    register_gate,
     register_head,
     register_mixer,
     register_norm,
     register_position,
 )
 from .norms import Normed, as_tensor  # noqa: F401
-from . import attention, block, embeddings, feedforward, head, norms  # noqa: F401  (register themselves)
+from . import attention, block, conv, embeddings, feedforward, head, latent_attention, norms, routed  # noqa: F401  (register themselves)

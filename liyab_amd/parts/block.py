@@ -4,6 +4,7 @@ from __future__ import annotations
 
 import torch
 
+from ..kernels import ops
 from .base import SplitStream, StepContext, settled
 from .registry import register_block
 
@@ -68,3 +69,68 @@ class PreNormBlock:
 
 
 register_block("pre_norm", PreNormBlock)
+
+
+class PostNormGatedBlock:
+    """x += norm_mixer(g1 * mixer(conv(x))); x += norm_ffn(g2 * ffn(x)): the sublayers read the stream
+    itself, and the norms stand on their results. g = sigmoid(W x + b) from the stream as the sublayer
+    gets it (before the convolution); `conv`: what the mixer reads is x + a short causal convolution of
+    x over time, whose last inputs are the layer's per-request state. Gates and the convolution are
+    optional, the feed-forward too. The sum into the stream, the norms and the gates are 32-bit; the
+    sublayers and the gates' products read x rounded to the compute dtype.
+
+    Kernels a sublayer beside its own: the convolution (which also rounds x), the gate's product, and
+    one update of the rows (sum of the sublayer's rows a token, gate, norm, addition, the rounded rows
+    for the next sublayer, and the rows the next step's convolution needs)."""
+
+    replayable = True
+    takes_padding_rows = True
+    takes_pending = False  # the stream is whole when this block gets it and when it leaves it
+
+    def __init__(self, spec, mixer, ffn, norm_mixer, norm_ffn, input_conv=None, gate_mixer=None, gate_ffn=None):
+        self.mixer, self.ffn, self.norm_mixer, self.norm_ffn = mixer, ffn, norm_mixer, norm_ffn
+        self.conv, self.gate_mixer, self.gate_ffn = input_conv, gate_mixer, gate_ffn if ffn is not None else None
+        self.dtype = mixer.dtype
+        self.mixer_phase = getattr(getattr(spec, "mixer", None), "kind", "mixer")
+        self.ffn_phase = getattr(getattr(spec, "ffn", None), "kind", "ffn")
+        for part, what in ((mixer, "mixer"), (ffn, "feed-forward")):
+            if part is not None and "out" not in part.forward.__code__.co_varnames:
+                raise ValueError(f"a post-norm block needs a {what} that can leave its result to the block (forward(..., out=))")
+        for norm in (norm_mixer, norm_ffn if ffn is not None else norm_mixer):
+            if not getattr(norm, "root_mean_square", False):
+                raise ValueError("a post-norm block's row update applies a root-mean-square norm (kind 'rmsnorm')")
+        if mixer.state_spec() is not None and self.conv is not None and self.conv.state_spec() is not None:
+            raise ValueError("a mixer with state of its own under an input convolution: one state a layer")
+
+    def state_spec(self):
+        return (self.conv.state_spec() if self.conv is not None else None) or self.mixer.state_spec()
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, cache, state, writes_cache: bool = True):
+        ws, n, d = ctx.workspace, x.shape[0], x.shape[1]
+        if ctx.phases is not None:
+            ctx.phases.mark(self.mixer_phase)
+        xh = ws.get("stream_cast", (n, d), self.dtype)
+        conv_state = state if self.conv is not None and self.conv.state_spec() is not None else None
+        if self.conv is not None:
+            h = self.conv.forward(x, ctx, conv_state, cast_out=xh)
+        else:
+            ops.gather_rows(xh, x)
+            h = xh
+        gate = self.gate_mixer.forward(xh, ctx, "gate_logits") if self.gate_mixer is not None else None
+        y = ws.get("sublayer_out", (n, d), torch.float32)
+        self.mixer.forward(h, ctx, cache, None if conv_state is not None else state, None, writes_cache=writes_cache, out=y)
+        keep = (conv_state, ctx) if conv_state is not None and writes_cache else None
+        ops.gated_norm_add(x, y, self.norm_mixer.weight, self.norm_mixer.eps, gate=gate, cast_out=xh if self.ffn is not None else None,
+                           keep=keep)
+        if self.ffn is not None:
+            if ctx.phases is not None:
+                ctx.phases.mark(self.ffn_phase)
+            gate = self.gate_ffn.forward(xh, ctx, "gate_logits") if self.gate_ffn is not None else None
+            k = int(getattr(self.ffn, "rows_a_token", 1))
+            y = ws.get("sublayer_rows", (n * k, d), torch.float32) if k > 1 else y
+            self.ffn.forward(xh, ctx, None, out=y)
+            ops.gated_norm_add(x, y, self.norm_ffn.weight, self.norm_ffn.eps, n_sum=k, gate=gate)
+        return None
+
+
+register_block("post_norm_gated", PostNormGatedBlock)

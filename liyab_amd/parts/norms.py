@@ -82,3 +82,31 @@ class LayerNorm:
 
 
 register_norm("layernorm", LayerNorm)
+
+
+class RMSNorm:
+    """y = x / sqrt(mean(x^2) + eps) * weight over the last axis, the epsilon inside the root; sums and
+    scaling 32-bit. `rows` gathers (the final norm runs on the wanted rows only). Behind a sublayer,
+    a block applies it through the fused residual update (`ops.gated_norm_add`), which reads
+    `weight` and `eps` from here."""
+
+    replayable = True
+    takes_padding_rows = True
+    root_mean_square = True  # (what `ops.gated_norm_add` applies, given this part's weight and eps)
+
+    def __init__(self, spec, store, dtype: torch.dtype):
+        self.width = spec.width
+        self.eps = float(spec.eps)
+        self.dtype = dtype
+        w = spec.tensors.get("weight")
+        self.weight = store.fetch(w, (self.width,), "vector") if w is not None else None
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, rows: Optional[torch.Tensor] = None,
+                n_rows: Optional[int] = None, name: str = "normed") -> torch.Tensor:
+        n = x.shape[-2] if rows is None else (n_rows if n_rows is not None else rows.numel())
+        out = ctx.workspace.get(name, (n, self.width), self.dtype)
+        ops.rmsnorm(out, x, self.weight, self.eps, rows=rows)
+        return out
+
+
+register_norm("rmsnorm", RMSNorm)

@@ -14,6 +14,7 @@ from ..errors import Unsupported
 
 _REGISTRIES: Dict[str, Dict[str, type]] = {
     "mixer": {}, "ffn": {}, "norm": {}, "position": {}, "block": {}, "embedding": {}, "head": {},
+    "conv": {}, "gate": {},
 }
 
 
@@ -29,6 +30,8 @@ def register_position(kind: str, cls: type) -> type: return _register("position"
 def register_block(kind: str, cls: type) -> type: return _register("block", kind, cls)
 def register_embedding(kind: str, cls: type) -> type: return _register("embedding", kind, cls)
 def register_head(kind: str, cls: type) -> type: return _register("head", kind, cls)
+def register_conv(kind: str, cls: type) -> type: return _register("conv", kind, cls)
+def register_gate(kind: str, cls: type) -> type: return _register("gate", kind, cls)
 
 
 def find_part(family: str, kind: str) -> type:

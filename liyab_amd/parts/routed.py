@@ -1,0 +1,64 @@
+"""A feed-forward that routes each token to a few of many experts."""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..kernels import ops
+from .base import StepContext, settled
+from .linear import linear
+from .norms import as_tensor
+from .registry import register_ffn
+
+
+class RoutedFFN:
+    """z = Wr h + b (32-bit sums, kept in 32 bits); a token takes the `top` experts with the largest z,
+    weighted by the softmax over those logits alone; expert e gives Wdown_e (silu(Wgate_e h) * (Wup_e
+    h)); the result is the weighted sum. The step's (token, choice) entries are listed by expert in
+    tiles, and two grouped products run over the tiles: [gate | up] with the activation, then down
+    with the router's weight; an entry's row is added to the others of its token by the reader."""
+
+    replayable = True
+    takes_padding_rows = True  # (they are routed and computed like token 0; nobody reads them)
+
+    def __init__(self, spec, store, dtype: torch.dtype):
+        self.dtype = dtype
+        self.width, self.inner, self.n_experts, self.top = spec.width, spec.inner, spec.n_experts, spec.top
+        if spec.activation != "silu":
+            raise ValueError(f"routed feed-forward: unknown activation '{spec.activation}'")
+        if not 1 <= self.top <= min(self.n_experts, ops.MOE_MAX_TOP):
+            raise ValueError(f"routed feed-forward: {self.top} of {self.n_experts} experts a token (at most {ops.MOE_MAX_TOP})")
+        t, E, F, d = spec.tensors, self.n_experts, self.inner, self.width
+        self.router = store.fetch(t["router"], (E, d), "matrix")
+        self.router_bias = store.fetch(t["router_bias"], (E,), "vector") if "router_bias" in t else None
+        self.gate = store.fetch_joined([t[("gate", e)] for e in range(E)], [(F, d)] * E, "matrix", "stack")
+        self.up = store.fetch_joined([t[("up", e)] for e in range(E)], [(F, d)] * E, "matrix", "stack")
+        self.down = store.fetch_joined([t[("down", e)] for e in range(E)], [(d, F)] * E, "matrix", "stack")
+
+    rows_a_token = property(lambda self: self.top)  # rows `forward(..., out=)` leaves for each token
+
+    def forward(self, h, ctx: StepContext, residual: Optional[torch.Tensor], out: Optional[torch.Tensor] = None):
+        """Adds the result into `residual`, or, with `out` (float32 [n * top, width]), leaves each token's
+        `top` weighted expert outputs there in consecutive rows, for a reader that adds them up."""
+        h = as_tensor(h)
+        n, ws, E, top = h.shape[0], ctx.workspace, self.n_experts, self.top
+        logits = ws.get("router_logits", (n, E), torch.float32)
+        linear(h, self.router, self.router_bias, out=logits)
+        tiles = ops.moe_tiles(n * top, E)
+        ids = ws.get("routed_ids", (n * top,), torch.int32)
+        weights = ws.get("routed_weights", (n * top,), torch.float32)
+        rows_list = ws.get("routed_rows", (tiles * ops.GROUPED_ROWS,), torch.int32)
+        tile_group = ws.get("routed_tiles", (tiles,), torch.int32)
+        ops.moe_route(logits, top, ids, weights, rows_list, tile_group)
+        inner = ws.get("routed_inner", (n * top, self.inner), self.dtype)
+        ops.moe_product(inner, h, self.gate, self.up, rows_list, tile_group, a_div=top)
+        y = out if out is not None else ws.get("routed_out", (n * top, self.width), torch.float32)
+        ops.moe_product(y, inner, self.down, None, rows_list, tile_group, row_scale=weights)
+        if out is None:
+            ops.gated_norm_add(settled(residual), y, None, 0.0, n_sum=top, normalize=False)
+        return None
+
+
+register_ffn("routed_ffn", RoutedFFN)

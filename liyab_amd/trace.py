@@ -50,7 +50,7 @@ def main(argv=None) -> int:
     from .engine import EngineCore, StepItem
 
     core = EngineCore(args.model, dtype=args.dtype, device=args.device, page_size=args.page_size,
-                      max_tokens=args.max_tokens, max_requests=16)
+                      max_tokens=args.max_tokens, max_requests=4)
     for line in sys.stdin:
         line = line.strip()
         if not line:

@@ -49,6 +49,7 @@ class WeightStore:
         self._missing: List[str] = []
         self._wrong: List[str] = []
         self._cache: Dict[Tuple[str, str, str], torch.Tensor] = {}
+        self._derived: Dict[tuple, torch.Tensor] = {}
 
     # -- construction -----------------------------------------------------
     @classmethod
@@ -70,7 +71,27 @@ class WeightStore:
     def has(self, src: TensorSource) -> bool:
         return self._resolve(src.name) is not None
 
-    def fetch(self, src: TensorSource, shape: Sequence[int], role: str) -> Optional[torch.Tensor]:
+    def fetch_joined(self, srcs: Sequence[TensorSource], shapes: Sequence[Sequence[int]], role: str, how: str = "rows") -> torch.Tensor:
+        """Several tensors of the file as one on the device: how = "rows", one after the other along their
+        first axis (projections of one input that run as one product), or "stack", along a new first axis
+        (the matrices of a layer's experts). The parts are not kept on their own; asked for again with the
+        same names, the same device tensor comes back (layers that share their weights share it)."""
+        key = (how, role) + tuple((s.name, s.layout) for s in srcs)
+        hit = self._derived.get(key)
+        if hit is None:
+            parts = [self.fetch(src, shape, role, keep=False) for src, shape in zip(srcs, shapes)]
+            hit = self._derived[key] = (torch.cat(parts, dim=0) if how == "rows" else torch.stack(parts, dim=0)).contiguous()
+        return hit
+
+    def derived(self, key: tuple, make) -> torch.Tensor:
+        """A tensor a part makes of its fetched ones once (another layout of a matrix), kept under `key`
+        (which names what it was made of) so that layers sharing their weights share it too."""
+        hit = self._derived.get(key)
+        if hit is None:
+            hit = self._derived[key] = make()
+        return hit
+
+    def fetch(self, src: TensorSource, shape: Sequence[int], role: str, keep: bool = True) -> Optional[torch.Tensor]:
         """The tensor `src` names, on the device, in working layout and dtype.
 
         `shape` is the working shape ("out_in" for matrices); `role` is
@@ -109,7 +130,8 @@ class WeightStore:
         if src.layout == "in_out":
             dev = dev.t()
         dev = dev.to(dtype).contiguous()
-        self._cache[key] = dev
+        if keep:
+            self._cache[key] = dev
         return dev
 
     def _dtype_for(self, role: str, stored: torch.dtype, name: str) -> Optional[torch.dtype]:

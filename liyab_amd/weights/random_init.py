@@ -76,6 +76,13 @@ class DrawingStore:
             raise ValueError(f"random weights: '{src.name}' is asked for as {list(stored)} and as {list(t.shape)}")
         return t.t() if src.layout == "in_out" else t
 
+    def fetch_joined(self, srcs, shapes, role: str, how: str = "rows") -> torch.Tensor:
+        parts = [self.fetch(src, shape, role) for src, shape in zip(srcs, shapes)]
+        return torch.cat(parts, dim=0) if how == "rows" else torch.stack(parts, dim=0)
+
+    def derived(self, key: tuple, make) -> torch.Tensor:
+        return make()
+
     def finish(self) -> None:
         pass
 
