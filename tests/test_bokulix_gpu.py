@@ -1,0 +1,561 @@
+"""Bokulix through the engine against its plain twin (`plain_bokulix.py`): each mechanism alone, then whole
+models of several geometries under every way of cutting and batching the work, in 32-bit and in bfloat16
+(needs the GPU). The geometries differ from each other in every size; one has sizes no kernel tiles
+evenly, one experts a token, as many experts as choices, one head, two taps and a layer without a window."""
+
+import json
+import math
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import plain_bokulix as plain
+import trace_tools as tt
+from conftest import ROOT, TOL
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DTYPES = ["float32", "bfloat16"]
+# Relative to the largest |logit| of the compared row, fixed. float32: the families below show 2.5e-6 to
+# 3.8e-6. bfloat16 against the twin in float64 with the same rounded matrices: 4.5e-2 to 5.6e-2, alike
+# whole, in portions, decoded and mixed (a norm stands on every sublayer's result and brings each
+# rounding of a sublayer back to the stream's own size, layer after layer, and these random models'
+# logits lie close together); the tolerance is one and a half times the largest.
+TOL_B = {"float32": TOL["float32"], "bfloat16": 8e-2}
+
+
+def mixer(heads, dim, vdim, rank, window, scale=None):
+    m = {"heads": heads, "dim": dim, "vdim": vdim, "kv_rank": rank, "scale": scale if scale is not None else 1.0 / math.sqrt(dim)}
+    if window:
+        m["mask"] = {"size": window}
+    return m
+
+
+def moe(experts, top, ff):
+    return {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}}
+
+
+def layer(m, mlp, weights_of=None):
+    entry = {"type": "latent_attention", "mixer": m, "mlp": mlp}
+    if weights_of is not None:
+        entry["weights_of"] = weights_of
+    return entry
+
+
+def config(vocab, width, positions, eps, taps, layers):
+    return {"architecture": "Bokulix", "vocab": vocab, "width": width, "max_positions": positions, "norm": {"eps": eps},
+            "canon": {"taps": taps}, "layers": layers}
+
+
+_E = mixer(4, 16, 24, 32, 24)
+_O = mixer(1, 12, 12, 20, 0)
+CONFIGS = {
+    # even sizes; a layer without a feed-forward and with a short window; two layers that run with the
+    # first one's tensors, one of them under a window of its own
+    "even": (config(300, 128, 512, 1e-6, 3, [layer(_E, moe(8, 2, 64)), layer(mixer(2, 32, 16, 64, 9), None),
+                                            layer(_E, moe(8, 2, 64), weights_of=0), layer(dict(_E, mask={"size": 70}), moe(8, 2, 64), weights_of=0)]), 11),
+    # sizes that no kernel tiles evenly: width 100, one head, rows of 20, a feed-forward of 50; one expert a
+    # token of three, then three of three; two taps; no window, then a window of one (a token sees itself)
+    "odd": (config(211, 100, 300, 1e-5, 2, [layer(_O, moe(3, 1, 50)), layer(dict(_O, mask={"size": 1}), moe(3, 3, 50)),
+                                            layer(mixer(3, 8, 40, 24, 33), moe(5, 4, 24))]), 12),
+    # five taps, one expert in all, a window past the context
+    "taps": (config(128, 64, 400, 1e-5, 5, [layer(mixer(2, 16, 16, 16, 1000), moe(1, 1, 32)), layer(mixer(8, 8, 8, 48, 17), moe(6, 2, 40))]), 13),
+}
+
+
+def every_expert(cfg):
+    """The same geometry with every expert chosen by every token. A choice among experts is a step in the
+    logits: a bfloat16 rounding on the way to a router whose two candidates lie a rounding apart takes
+    the other expert, and the row differs by far more than any rounding (in these random models about one
+    token in a hundred a layer). Whole models are therefore compared in bfloat16 with routers that weigh
+    all experts, which is continuous; the choice itself is compared in 32-bit throughout and, in
+    bfloat16, in the tests of the routing and of the routed products alone."""
+    cfg = json.loads(json.dumps(cfg))
+    for entry in cfg["layers"]:
+        if entry["mlp"] is not None:
+            entry["mlp"]["router"]["top"] = entry["mlp"]["router"]["experts"]
+    return cfg
+
+
+def config_of(name, dtype):
+    cfg, seed = CONFIGS[name]
+    return (every_expert(cfg) if dtype == "bfloat16" else cfg), seed
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    """{(name, dtype): (folder, config, float64 tensors as that path holds them)}, float32 files written by
+    the random-weights mode."""
+    from liyab_amd.weights import write_random_model
+
+    out = {}
+    for name in CONFIGS:
+        for dtype in DTYPES:
+            cfg, seed = config_of(name, dtype)
+            d = str(tmp_path_factory.mktemp(f"bokulix_{name}_{dtype}"))
+            write_random_model(d, json.loads(json.dumps(cfg)), seed)
+            raw, tensors = plain.read_model(d)
+            out[(name, dtype)] = (d, raw, twin_tensors(tensors, dtype))
+    return out
+
+
+def twin_tensors(tensors, dtype):
+    return tensors if dtype == "float32" else plain.round_matrices(tensors)
+
+
+def make_requests(name):
+    cfg, seed = CONFIGS[name]
+    V, P = cfg["vocab"], cfg["max_positions"]
+    lens = {"even": [1, 2, 23, 70, 131, 260], "odd": [3, 40, 97, 200], "taps": [4, 5, 66, 150]}[name]
+    return {f"{name}{i}": tt.random_tokens(seed * 50 + i, n, V) for i, n in enumerate(lens)}
+
+
+@pytest.fixture(scope="module")
+def reference(models):
+    return {(name, dtype): {rid: plain.forward(raw, t, toks) for rid, toks in make_requests(name).items()}
+            for (name, dtype), (_, raw, t) in models.items()}
+
+
+def make_core(model_dir, dtype, max_tokens, page_size=16, max_requests=4, **kw):
+    from liyab_amd.engine import EngineCore
+
+    core = EngineCore(model_dir, dtype=dtype, page_size=page_size, max_tokens=max_tokens, max_requests=max_requests, **kw)
+    # free pages and unused state hold NaN: a kernel that reads past a request's length, or a slot's old
+    # rows, shows it
+    for c in core.storage.layers.values():
+        for t in c.rows.values():
+            t.fill_(float("nan"))
+    for t in core.storage.states.values():
+        t.fill_(float("nan"))
+    torch.cuda.synchronize()
+    return core
+
+
+# ---------------------------------------------------------------------------
+# each mechanism alone
+# ---------------------------------------------------------------------------
+def rand(rng, *shape, scale=1.0, mean=0.0):
+    return torch.from_numpy((rng.standard_normal(shape) * scale + mean).astype(np.float32))
+
+
+def f64(t):
+    return t.detach().float().cpu().numpy().astype(np.float64)
+
+
+@pytest.mark.parametrize("d", [96, 100, 2500])
+def test_norm_and_row_update_alone(d):
+    from liyab_amd.kernels import ops
+
+    rng = np.random.default_rng(1)
+    x, w = rand(rng, 7, d, scale=2.0, mean=0.3).to(DEV), rand(rng, d, scale=0.2, mean=1.0).to(DEV)
+    rows = torch.tensor([5, 0, 5], dtype=torch.int32, device=DEV)
+    for dt, tol in ((torch.float32, 1e-6), (torch.bfloat16, 5e-3)):
+        out = torch.empty(3, d, dtype=dt, device=DEV)
+        ops.rmsnorm(out, x, w, 1e-3, rows=rows)
+        assert tt.rel_err(f64(out), plain.rms(f64(x)[[5, 0, 5]], f64(w), 1e-3)) < tol
+    # the update of the rows: three rows a token added up, a gate whose logits are columns of a wider
+    # tensor, the norm, the sum into the stream, and the rounded copy
+    y, wide = rand(rng, 21, d, scale=3.0).to(DEV), rand(rng, 7, d + 9, scale=2.0).to(DEV)
+    gate = wide[:, 4:4 + d]
+    s = f64(y).reshape(7, 3, d).sum(1) * plain.sigmoid(f64(gate))
+    want = f64(x) + plain.rms(s, f64(w), 1e-5)
+    x1, cast = x.clone(), torch.empty(7, d, dtype=torch.bfloat16, device=DEV)
+    ops.gated_norm_add(x1, y, w, 1e-5, n_sum=3, gate=gate, cast_out=cast)
+    assert tt.rel_err(f64(x1), want) < 1e-6
+    assert torch.equal(cast, x1.to(torch.bfloat16))
+    x2 = x.clone()
+    ops.gated_norm_add(x2, y[:7], None, 1e-5)  # no gate, no weight
+    assert tt.rel_err(f64(x2), f64(x) + plain.rms(f64(y[:7]), 1.0, 1e-5)) < 1e-6
+    x3 = x.clone()
+    ops.gated_norm_add(x3, y, None, 0.0, n_sum=3, normalize=False)  # the plain sum of a token's rows
+    assert tt.rel_err(f64(x3), f64(x) + f64(y).reshape(7, 3, d).sum(1)) < 1e-6
+
+
+@pytest.mark.parametrize("shape", [(4, 16, 32), (3, 40, 24), (1, 12, 20), (5, 20, 13)])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_products_a_head_alone(dtype, shape):
+    """out[t, h] = a[t, h] . w[h]^T for every head, operands that are column ranges of wider rows, with and
+    without a gate; sizes the matrix cores take and sizes they do not."""
+    from liyab_amd.kernels import ops
+
+    H, N, K = shape
+    dt = torch.float32 if dtype == "float32" else torch.bfloat16
+    rng = np.random.default_rng(2)
+    for n in (1, 5, 64, 131):
+        wide = rand(rng, n, H * K + 16).to(dt).to(DEV)
+        a = wide[:, 8:8 + H * K]
+        w = rand(rng, H, N, K).to(dt).to(DEV)
+        glog = rand(rng, n, H * N + 3, scale=2.0).to(dt).to(DEV)[:, 3:]
+        want = np.einsum("nhk,hjk->nhj", f64(a).reshape(n, H, K), f64(w)).reshape(n, H * N)
+        out = torch.full((n, H * N), float("nan"), dtype=dt, device=DEV)
+        ops.heads_product(out, a, w)
+        assert tt.rel_err(f64(out), want) < (1e-6 if dtype == "float32" else 6e-3)
+        out32 = torch.empty(n, H * N, dtype=torch.float32, device=DEV)
+        ops.heads_product(out32, a, w, gate=glog)
+        assert tt.rel_err(f64(out32), want * plain.sigmoid(f64(glog))) < (1e-6 if dtype == "float32" else 1e-5)
+
+
+@pytest.mark.parametrize("experts,top", [(8, 2), (3, 3), (5, 1), (64, 6)])
+@pytest.mark.parametrize("n", [1, 7, 300])
+def test_routing_alone(experts, top, n):
+    """The chosen experts and their weights against the twin's; every (token, choice) entry stands exactly
+    once in its expert's tiles, tiles no expert uses are marked, and equal logits go to the lower number."""
+    from liyab_amd.kernels import ops
+
+    rng = np.random.default_rng(3)
+    logits = rand(rng, n, experts + 5, scale=3.0).to(DEV)[:, 2:2 + experts]
+    logits[0, :] = 0.25  # all equal: the first `top` experts
+    tiles = ops.moe_tiles(n * top, experts)
+    ids = torch.empty(n * top, dtype=torch.int32, device=DEV)
+    weights = torch.empty(n * top, dtype=torch.float32, device=DEV)
+    rows_list = torch.full((tiles * ops.GROUPED_ROWS,), -7, dtype=torch.int32, device=DEV)
+    tile_group = torch.full((tiles,), -7, dtype=torch.int32, device=DEV)
+    ops.moe_route(logits, top, ids, weights, rows_list, tile_group)
+    z = f64(logits)
+    order = np.argsort(-z, axis=-1, kind="stable")[:, :top]
+    chosen = np.take_along_axis(z, order, -1)
+    w = np.exp(chosen - chosen.max(-1, keepdims=True))
+    w /= w.sum(-1, keepdims=True)
+    assert np.array_equal(ids.cpu().numpy().reshape(n, top), order)
+    assert np.abs(f64(weights).reshape(n, top) - w).max() < 1e-6
+    listed, groups = rows_list.cpu().numpy().reshape(tiles, -1), tile_group.cpu().numpy()
+    flat_ids = ids.cpu().numpy()
+    seen = []
+    for tile in range(tiles):
+        if groups[tile] < 0:
+            assert (listed[tile] == -1).all()
+            continue
+        entries = listed[tile][listed[tile] >= 0]
+        assert len(entries) and (flat_ids[entries] == groups[tile]).all()
+        seen += entries.tolist()
+    assert sorted(seen) == list(range(n * top))
+
+
+@pytest.mark.parametrize("sizes", [(8, 2, 64, 96), (3, 3, 50, 100), (6, 1, 24, 40)])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_routed_products_alone(dtype, sizes):
+    """The two grouped products over the routed entries against a loop over tokens and choices."""
+    from liyab_amd.kernels import ops
+
+    E, top, F, d = sizes
+    dt = torch.float32 if dtype == "float32" else torch.bfloat16
+    rng = np.random.default_rng(4)
+    for n in (1, 9, 150):
+        h = rand(rng, n, d).to(dt).to(DEV)
+        wg, wu = rand(rng, E, F, d, scale=d ** -0.5).to(dt).to(DEV), rand(rng, E, F, d, scale=d ** -0.5).to(dt).to(DEV)
+        wd = rand(rng, E, d, F, scale=F ** -0.5).to(dt).to(DEV)
+        logits = rand(rng, n, E, scale=2.0).to(DEV)
+        tiles = ops.moe_tiles(n * top, E)
+        ids, weights = torch.empty(n * top, dtype=torch.int32, device=DEV), torch.empty(n * top, dtype=torch.float32, device=DEV)
+        rows_list, tile_group = torch.empty(tiles * ops.GROUPED_ROWS, dtype=torch.int32, device=DEV), torch.empty(tiles, dtype=torch.int32, device=DEV)
+        ops.moe_route(logits, top, ids, weights, rows_list, tile_group)
+        inner = torch.full((n * top, F), float("nan"), dtype=dt, device=DEV)
+        ops.moe_product(inner, h, wg, wu, rows_list, tile_group, a_div=top)
+        out = torch.full((n * top, d), float("nan"), dtype=torch.float32, device=DEV)
+        ops.moe_product(out, inner, wd, None, rows_list, tile_group, row_scale=weights)
+        hi, e_of, w_of = f64(h), ids.cpu().numpy(), f64(weights)
+        want_inner, want = np.zeros((n * top, F)), np.zeros((n * top, d))
+        for entry in range(n * top):
+            e, x = e_of[entry], hi[entry // top]
+            g = f64(wg[e]) @ x
+            want_inner[entry] = g * plain.sigmoid(g) * (f64(wu[e]) @ x)
+            want[entry] = w_of[entry] * (f64(wd[e]) @ f64(inner[entry]))
+        assert tt.rel_err(f64(inner), want_inner) < (2e-6 if dtype == "float32" else 8e-3)
+        assert tt.rel_err(f64(out), want) < (2e-6 if dtype == "float32" else 2e-5)
+
+
+class _Layer:
+    """A one-layer engine whose step context, cache and state the mechanism tests borrow."""
+
+    def __init__(self, dtype, m, taps=4, width=64, mlp=None, tensors=None, page_size=8):
+        from liyab_amd.config import config_from_dict
+        from liyab_amd.engine import EngineCore
+        from liyab_amd.weights.random_init import random_tensors
+
+        self.raw = config(50, width, 2048, 1e-5, taps, [layer(m, mlp)])
+        cfg = config_from_dict(self.raw)
+        t = random_tensors(cfg, 5)
+        t.update(tensors or {})
+        if dtype == "bfloat16":
+            t = {k: (v.to(torch.bfloat16).float() if v.dim() == 2 and not k.endswith("canon1") else v) for k, v in t.items()}
+        self.t = {k: f64(v) for k, v in t.items()}
+        self.core = EngineCore.from_plan(cfg.plan(), t, dtype=dtype, page_size=page_size, num_pages=300, max_requests=3, use_graphs=False)
+        for s in self.core.storage.states.values():
+            s.fill_(float("nan"))
+        self.block = self.core.model.blocks[0]
+        self.width, self.dtype = width, dtype
+
+    def run(self, rid, rows, portions, fn):
+        """Feeds `rows` [n, width] of request `rid` in `portions`; fn(ctx, rows of the portion) -> what it computed."""
+        from liyab_amd.engine import StepItem
+
+        out, done = [], 0
+        for take in portions:
+            item = StepItem(rid, [1] * take, [])
+            ctx, lengths = self.core.step_fn.prepare([item])
+            out.append(fn(ctx, rows[done:done + take].to(DEV)))
+            self.core.step_fn.commit([item], lengths)
+            done += take
+        assert done == rows.shape[0]
+        return np.concatenate(out)
+
+
+@pytest.mark.parametrize("taps", [1, 2, 4, 7])
+def test_input_convolution_alone_in_portions(taps):
+    """Portions down to one token read what earlier portions left in the request's state; a second
+    request in a slot that was used before starts from zeros, whatever the slot still holds."""
+    p = _Layer("float32", mixer(2, 8, 8, 16, 0), taps=taps)
+    conv, core = p.block.conv, p.core
+    state = core.storage.state(0)
+    assert (state is None) == (taps == 1)
+    rng = np.random.default_rng(6)
+    for rid, portions in (("a", (9, 1, 1, 2, 1, 5, 3, 1, 1, 1, 17)), ("b", (1, 1, 2, 30)), ("c", (41,))):
+        core.open(rid)
+        x = rand(rng, sum(portions), p.width, scale=1.5)
+
+        def step(ctx, xs):
+            out = conv.forward(xs, ctx, state)
+            conv.keep(xs, ctx, state)
+            return f64(out)
+
+        got = p.run(rid, x, portions, step)
+        assert tt.rel_err(got, plain.input_convolution(f64(x), p.t["l0.canon1"])) < 1e-6, (rid, taps)
+        core.close(rid)
+
+
+def _mixer_alone(p, x, portions, rid="m"):
+    core, mix = p.core, p.block.mixer
+    core.open(rid)
+
+    def step(ctx, xs):
+        h = xs.to(core.dtype)
+        y = torch.empty(xs.shape[0], p.width, dtype=torch.float32, device=DEV)
+        mix.forward(h, ctx, core.storage.layer(0), None, None, out=y)
+        base = torch.ones(xs.shape[0], p.width, device=DEV)
+        mix.forward(h, ctx, core.storage.layer(0), None, base, writes_cache=False)  # the other way to hand the result over
+        assert tt.rel_err(f64(base) - 1.0, f64(y)) < 1e-5
+        return f64(y)
+
+    got = p.run(rid, x, portions, step)
+    core.close(rid)
+    core.manager.check()
+    return got
+
+
+@pytest.mark.parametrize("m", [mixer(4, 16, 24, 32, 0), mixer(3, 8, 40, 24, 13), mixer(1, 12, 12, 20, 5), mixer(2, 32, 16, 128, 40)])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_latent_attention_alone(dtype, m):
+    """The mixer over its own cached rows: a portion, then more portions and single tokens, against the twin,
+    which makes every position's keys and values."""
+    p = _Layer(dtype, m)
+    x = rand(np.random.default_rng(7), 75, p.width, scale=1.2)
+    xs = x.to(torch.bfloat16).float() if dtype == "bfloat16" else x
+    want = plain.latent_attention(f64(xs), p.t, "l0.mix.", m, 1e-5)
+    got = _mixer_alone(p, x, (25, 1, 9, 1, 1, 2, 36))
+    assert tt.rel_err(got, want) < (1e-5 if dtype == "float32" else 1.5e-2)
+
+
+def _marked_tensors(width, H, D, V, R):
+    """Weights under which a query finds the keys that lie along its own input: the cached row is the
+    input's first R channels (normalised), a head's key its first D of them, a head's query the same
+    channels of the input, and values come from the other channels of the cached row."""
+    eye = torch.eye(width)
+    t = {"l0.mix.dkv": eye[:R].clone(), "l0.mix.dkv.norm": torch.ones(R)}
+    t["l0.mix.q"] = torch.cat([eye[:D]] * H).clone()
+    t["l0.mix.uk"] = torch.cat([torch.eye(R)[:D]] * H).clone()
+    uv = torch.zeros(H * V, R)
+    for h in range(H):
+        for e in range(V):
+            uv[h * V + e, D + (h + e) % (R - D)] = 1.0 + 0.1 * h
+    t["l0.mix.uv"] = uv
+    t["l0.mix.g"] = torch.zeros(H * V, width)
+    return t
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("window,page_size", [(0, 8), (40, 8), (33, 16)])
+def test_a_marked_key_far_away_and_at_the_windows_edge(dtype, window, page_size):
+    """One earlier position carries the query's own direction and a value of its own; the scores are scaled
+    so that it and the query's own position share nearly all the weight. Whether the query sees it is then
+    most of its output: far back among hundreds (no window), just inside and just outside the window, at
+    page borders, as the last token of a prompt's portion and decoded alone."""
+    # (48 dimensions a key: a key along the query scores 48 x 0.7, a random one 0.7 x N(0, 48), so that
+    # hundreds of random keys together weigh nothing beside one that is aligned)
+    H, D, V, R, width = 2, 48, 6, 64, 64
+    m = mixer(H, D, V, R, window, scale=0.7)
+    p = _Layer(dtype, m, width=width, tensors=_marked_tensors(width, H, D, V, R), page_size=page_size)
+    rng = np.random.default_rng(8)
+    n = 330
+    query_at = [n - 1, n - 2, 290, 2 * page_size * 8 + 1]
+    for case, distance in enumerate([window - 1, window, window + 1, 1] if window else [n - 4, 200, 257, n - 1 - page_size]):
+        x = rand(rng, n, width, scale=1.0)
+        marks = {}
+        for i in query_at:
+            j = i - distance
+            if j < 0 or j in marks or j in query_at or any(abs(j - o) < 2 for o in marks):
+                continue
+            marks[j] = i
+            x[j, :D] = 4.0 * x[i, :D]  # the same direction: its key matches query i as well as i's own
+            x[j, D:R] = rand(rng, R - D, scale=3.0)  # and a value of its own
+        xs = x.to(torch.bfloat16).float() if dtype == "bfloat16" else x
+        want = plain.latent_attention(f64(xs), p.t, "l0.mix.", m, 1e-5)
+        # the mark matters: without it the marked queries' outputs are far from what they are with it
+        blind = f64(xs).copy()
+        for j in marks:
+            blind[j] = 0.01
+        moved = np.abs(plain.latent_attention(blind, p.t, "l0.mix.", m, 1e-5) - want)[list(marks.values())].max(-1)
+        visible = window == 0 or distance < window
+        assert (moved > 0.3).all() if visible else (moved < 1e-6).all(), (window, distance, moved)
+        tol = 1e-5 if dtype == "float32" else 6e-2
+        for portions in ((n,), (n - 40,) + (1,) * 40, (100, 2, 150, 37, 2, 37, 2)):
+            got = _mixer_alone(p, x, portions, rid=f"m{case}")
+            assert tt.rel_err(got, want) < tol, (window, distance, portions[:3])
+
+
+# ---------------------------------------------------------------------------
+# whole models
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_each_request_alone_and_whole_and_every_layer(name, dtype, models, reference):
+    reqs = make_requests(name)
+    steps = tt.schedule_whole(reqs)
+    core = make_core(models[(name, dtype)][0], dtype, tt.max_live_tokens(steps))
+    got = tt.run_schedule(core, steps)
+    tt.check_against_plain(got, reqs, reference[(name, dtype)], TOL_B[dtype], f"bokulix-whole {name} {dtype}")
+    core.manager.check()
+    assert core.manager.pages_in_use() == 0
+    if dtype == "float32":
+        # the residual stream after every layer of one request, against the twin's
+        from liyab_amd.engine import StepItem
+
+        rid, toks = list(reqs.items())[2]
+        streams, caught = [], []
+        plain.forward(models[(name, dtype)][1], models[(name, dtype)][2], toks, streams)
+        plain_core = make_core(models[(name, dtype)][0], dtype, 512, use_graphs=False)
+        plain_core.model.replay_layers = False
+        for block in plain_core.model.blocks:
+            def wrapped(x, ctx, cache, state, writes_cache=True, _f=block.forward):
+                out = _f(x, ctx, cache, state, writes_cache=writes_cache)
+                caught.append(f64(x)[:len(toks)])
+                return out
+            block.forward = wrapped
+        plain_core.open(rid)
+        plain_core.step([StepItem(rid, toks, [])])
+        for got_x, want_x in zip(caught, streams):
+            assert tt.rel_err(got_x, want_x) < 1e-5
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_a_prompt_then_its_last_tokens_one_by_one(name, dtype, models, reference):
+    reqs = make_requests(name)
+    steps = tt.schedule_bulk_tail(reqs, tail=45)  # past the shorter windows
+    core = make_core(models[(name, dtype)][0], dtype, tt.max_live_tokens(steps))
+    got = tt.run_schedule(core, steps)
+    tt.check_against_plain(got, reqs, reference[(name, dtype)], TOL_B[dtype], f"bokulix-decode {name} {dtype}")
+    assert core.manager.pages_in_use() == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("sizes", [(5, 2, 17, 3, 48, 2, 31, 7), (2, 2, 2, 3), (1, 64, 1, 16, 2)])
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_portions_of_changing_size(name, dtype, sizes, models, reference):
+    reqs = make_requests(name)
+    if sizes[0] == 2:
+        reqs = dict(list(reqs.items())[:3])
+    steps = tt.schedule_portions(reqs, sizes)
+    core = make_core(models[(name, dtype)][0], dtype, tt.max_live_tokens(steps), page_size=8 if sizes[0] == 1 else 16)
+    got = tt.run_schedule(core, steps)
+    tt.check_against_plain(got, reqs, reference[(name, dtype)], TOL_B[dtype], f"bokulix-portions {name} {dtype}")
+    assert core.manager.pages_in_use() == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("seed,max_live,page_size", [(0, 4, 16), (1, 3, 8), (2, 2, 24)])
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_mixed_batches_with_pages_and_slots_used_again(name, dtype, seed, max_live, page_size, models, reference):
+    """Up to `max_live` requests at a time, portions of some beside single tokens of others, in a pool
+    and with state slots just large enough: what a finished request gives back is used by the next."""
+    base = make_requests(name)
+    reqs = {f"{rid}#{k}": toks for k in range(2) for rid, toks in base.items()}  # each request twice: more turnover
+    ref = {f"{rid}#{k}": reference[(name, dtype)][rid] for k in range(2) for rid in base}
+    steps = tt.schedule_mixed(reqs, seed=seed, max_live=max_live)
+    core = make_core(models[(name, dtype)][0], dtype, None, page_size=page_size, max_requests=max_live, num_pages=tt.max_live_pages(steps, page_size))
+    got = tt.run_schedule(core, steps)
+    tt.check_against_plain(got, reqs, ref, TOL_B[dtype], f"bokulix-mixed {name} {dtype}")
+    core.manager.check()
+    assert core.manager.pages_in_use() == 0
+    assert core.step_fn.graph_replays > 0  # the decode-only steps of the tail were replayed from graphs
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_long_decoding_from_the_first_token(dtype, models, reference):
+    """Every token on its own from position 0 on, across all windows many times over."""
+    name = "even"
+    rid, toks = list(make_requests(name).items())[-1]
+    reqs = {rid: toks}
+    steps = tt.schedule_bulk_tail(reqs, tail=len(toks))
+    core = make_core(models[(name, dtype)][0], dtype, tt.max_live_tokens(steps))
+    got = tt.run_schedule(core, steps)
+    tt.check_against_plain(got, reqs, reference[(name, dtype)], TOL_B[dtype], f"bokulix-long {dtype}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_the_trace_program(dtype, models, reference, tmp_path):
+    name = "odd"
+    reqs = make_requests(name)
+    steps = tt.schedule_mixed(reqs, seed=5, max_live=4)
+    got = tt.run_trace_program(models[(name, dtype)][0], dtype, steps, str(tmp_path), tt.max_live_tokens(steps), CONFIGS[name][0]["vocab"])
+    tt.check_against_plain(got, reqs, reference[(name, dtype)], TOL_B[dtype], f"bokulix-trace {dtype}")
+
+
+def _near_argmax(row, token, tol):
+    return row[token] >= row.max() - tol * np.abs(row).max()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["even", "odd"])
+def test_greedy_generation_through_the_entry_point(name, dtype, models):
+    """Engine.generate: the scheduler batches the prompts in portions beside decoding requests, in a pool
+    that does not hold them all at once; each token is the twin's greedy choice given the tokens so far."""
+    from liyab_amd import Engine, SamplingParams
+
+    d, raw, t = models[(name, dtype)]
+    V = raw["vocab"]
+    prompts = [tt.random_tokens(70 + i, n, V) for i, n in enumerate([1, 13, 64, 100, 7])]
+    n_new = 20
+    engine = Engine(d, dtype=dtype, page_size=16, num_pages=14, max_num_seqs=3, max_batched_tokens=48, prefill_chunk=24)
+    engine.stop_at_eos = False
+    results = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=n_new))
+    for prompt, res in zip(prompts, results):
+        assert len(res.tokens) == n_new
+        ref = plain.forward(raw, t, prompt + res.tokens[:-1])
+        for i, tok in enumerate(res.tokens):
+            row = ref[len(prompt) - 1 + i]
+            assert _near_argmax(row, tok, TOL_B[dtype]), f"token {i} of prompt length {len(prompt)}: {tok} vs {int(np.argmax(row))}"
+        if dtype == "float32":
+            assert res.tokens == plain.generate_greedy(raw, t, prompt, n_new)
+    assert engine.core.manager.pages_in_use() == 0
+    engine.core.manager.check()
+
+
+def test_command_line(models):
+    d, raw, tensors = models[("taps", "float32")]
+    prompt = tt.random_tokens(90, 11, raw["vocab"])
+    p = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "liyab-cli"), "-m", d, "-p", ",".join(map(str, prompt)), "-n", "6",
+                        "--temp", "0", "--dtype", "float32", "--json"], capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    turn = [json.loads(l) for l in p.stdout.splitlines() if l.startswith("{")][1]
+    assert turn["tokens"] == plain.generate_greedy(raw, tensors, prompt, 6)
+    # per-phase device times name the design's parts
+    p2 = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "liyab-cli"), "-m", d, "-p", ",".join(map(str, prompt)), "-n", "6",
+                         "--temp", "0", "--dtype", "float32", "--json", "--phases"], capture_output=True, text=True, timeout=300)
+    assert p2.returncode == 0, p2.stderr[-2000:]
+    turn2 = [json.loads(l) for l in p2.stdout.splitlines() if l.startswith("{")][1]
+    assert turn2["tokens"] == turn["tokens"]
+    assert set(turn2["phases_ms"]) == {"embed", "latent_attention", "routed_ffn", "lm_head"}
