@@ -6,6 +6,7 @@
     python bench.py --workload medium16|xl64         # the continuous-batching and the batch-64 workloads of the larger sizes
     python bench.py --link-floor                     # what one dependent kernel of a replayed graph costs at least
     python bench.py --product 4096,4096,16384,8,15   # one product in tiles of 128 x 128 and of 256 x 256
+    python bench.py --design bokulix [--design-sizes small,medium,xl] [--layers L] [--phases]   # Bokulix beside GPT-2 at equal sizes
 
 The default run has GPT-2 small's layer sizes (12 layers, width 768, 12 heads
 of 64, feed-forward 3072, vocabulary 50257, 1024 positions) with random
@@ -77,8 +78,9 @@ def make_engine(model_dir, dtype, batch, ctx, page_size=64, prefill_chunk=1024, 
                   phases=phases)
 
 
-def decode_run(engine, cfg, batch, prompt_len, steps, warmup, seed=11):
-    """(tokens/s, ms/step, bytes/step) over `steps` decode steps of `batch` requests."""
+def decode_run(engine, cfg, batch, prompt_len, steps, warmup, seed=11, step_bytes=None):
+    """(tokens/s, ms/step, bytes/step) over `steps` decode steps of `batch` requests. `step_bytes(contexts, steps,
+    elt)`: the bytes a timed step has to read, for a design whose bytes are not GPT-2's."""
     import numpy as np
     import torch
 
@@ -87,7 +89,7 @@ def decode_run(engine, cfg, batch, prompt_len, steps, warmup, seed=11):
     rng = np.random.default_rng(seed)
     engine.stop_at_eos = False
     for i in range(batch):
-        prompt = rng.integers(0, cfg["vocab_size"], prompt_len).tolist()
+        prompt = rng.integers(0, cfg.get("vocab_size", cfg.get("vocab")), prompt_len).tolist()
         # (requests that go on for some steps past the timed ones: a request about to reach its last
         # token is waited for, not run ahead of, and that wait is no part of a decode step)
         engine.add_request(prompt, SamplingParams(temperature=0.0, max_tokens=steps + warmup + 8), rid=f"b{batch}-{i}")
@@ -105,7 +107,10 @@ def decode_run(engine, cfg, batch, prompt_len, steps, warmup, seed=11):
     elt = 2 if engine.core.dtype == torch.bfloat16 else 4
     # each timed step s reads the cache of positions [0, context + s] of every request
     kv_positions = sum(c * steps + steps * (steps + 1) // 2 for c in contexts)
-    bytes_per_step = weight_bytes(cfg, elt) + kv_positions * kv_bytes_per_position(cfg, elt) / max(steps, 1)
+    if step_bytes is not None:
+        bytes_per_step = step_bytes(contexts, steps, elt)
+    else:
+        bytes_per_step = weight_bytes(cfg, elt) + kv_positions * kv_bytes_per_position(cfg, elt) / max(steps, 1)
     for r in list(engine.scheduler.running):
         engine.abort(r.rid)
     return batch * steps / dt, dt * 1e3 / max(steps, 1), bytes_per_step
@@ -241,7 +246,7 @@ def prefill_run(engine, cfg, prompt_lens, repeat=5, seed=12):
     from liyab_amd.engine import StepItem
 
     rng = np.random.default_rng(seed)
-    prompts = [rng.integers(0, cfg["vocab_size"], n) for n in prompt_lens]  # arrays of ids, as the scheduler hands portions over
+    prompts = [rng.integers(0, cfg.get("vocab_size", cfg.get("vocab")), n) for n in prompt_lens]  # arrays of ids, as the scheduler hands portions over
     best = float("inf")
     for it in range(repeat + 2):
         for i in range(len(prompts)):
@@ -340,6 +345,108 @@ def sequences_run(engine, cfg, counts, prompt_len, n_new, seed=13):
     return {"metric": "sequences together against in turns", "prompt_len": prompt_len, "new_tokens": n_new, "runs": out}
 
 
+# -- Bokulix beside GPT-2 at equal sizes ------------------------------------------------------------------
+# Layers that resemble real ones: GPT-2 small's, medium's and XL's widths, head counts and feed-forward widths; the
+# Bokulix of each has the same width, layers, heads (of 64, values of 64), vocabulary and positions, a cached row
+# of 128 (256 at XL's width), a window that covers the context (so that attention walks as many keys), four taps,
+# and experts whose chosen ones together are as wide as GPT-2's feed-forward (top x ff = n_inner).
+BOKULIX_SHAPES = {"small": {"rank": 128, "experts": 8, "top": 2}, "medium": {"rank": 128, "experts": 16, "top": 2},
+                  "xl": {"rank": 256, "experts": 16, "top": 4}}
+
+
+def bokulix_config(gpt2_cfg, shape):
+    d, H, F, L = gpt2_cfg["n_embd"], gpt2_cfg["n_head"], gpt2_cfg["n_inner"], gpt2_cfg["n_layer"]
+    hd = d // H
+    entry = {"type": "latent_attention",
+             "mixer": {"heads": H, "dim": hd, "vdim": hd, "kv_rank": shape["rank"], "scale": hd ** -0.5, "mask": {"size": gpt2_cfg["n_positions"]}},
+             "mlp": {"kind": "moe", "expert": {"ff": F // shape["top"]}, "router": {"experts": shape["experts"], "top": shape["top"]}}}
+    return {"architecture": "Bokulix", "vocab": gpt2_cfg["vocab_size"], "width": d, "max_positions": gpt2_cfg["n_positions"],
+            "norm": {"eps": 1e-5}, "canon": {"taps": 4}, "layers": [json.loads(json.dumps(entry)) for _ in range(L)]}
+
+
+def bokulix_step_bytes(cfg, batch):
+    """The bytes a decode step of `batch` tokens has to read: every matrix of the mixers, gates and routers once, the
+    experts that tokens choose (as many distinct ones as uniform choices make on average), the head, and the cached rows
+    inside each request's window."""
+    def step_bytes(contexts, steps, elt):
+        d, V = cfg["width"], cfg["vocab"]
+        total = V * d * elt
+        for entry in cfg["layers"]:
+            m, mlp = entry["mixer"], entry["mlp"]
+            H, D, Vd, R = m["heads"], m["dim"], m["vdim"], m["kv_rank"]
+            total += ((H * D + R + H * Vd) * d + H * D * R + H * Vd * R + d * H * Vd + d * d) * elt
+            if mlp is not None:
+                E, top, F = mlp["router"]["experts"], mlp["router"]["top"], mlp["expert"]["ff"]
+                chosen = E * (1.0 - (1.0 - top / E) ** batch)
+                total += (d * d + E * d) * elt + chosen * 3 * F * d * elt
+            window = (m.get("mask") or {}).get("size", 0)
+            seen = sum(sum(min(c + s + 1, window) if window else c + s + 1 for s in range(steps)) for c in contexts) / max(steps, 1)
+            total += seen * R * elt
+        return total
+    return step_bytes
+
+
+def bokulix_prefill_flops(cfg, prompt_lens, logit_rows):
+    d, V, n = cfg["width"], cfg["vocab"], sum(prompt_lens)
+    flops = 2.0 * logit_rows * d * V
+    for entry in cfg["layers"]:
+        m, mlp = entry["mixer"], entry["mlp"]
+        H, D, Vd, R = m["heads"], m["dim"], m["vdim"], m["kv_rank"]
+        flops += 2.0 * n * ((H * D + R + H * Vd) * d + H * D * R + H * Vd * R + d * H * Vd + d * d)
+        window = (m.get("mask") or {}).get("size", 0)
+        for t in prompt_lens:
+            keys = sum(min(i + 1, window) if window else i + 1 for i in range(t))
+            flops += 4.0 * H * R * keys  # scores and weighted rows against the cached rows
+        if mlp is not None:
+            E, top, F = mlp["router"]["experts"], mlp["router"]["top"], mlp["expert"]["ff"]
+            flops += 2.0 * n * (d * d + E * d + top * 3 * F * d)
+    return flops
+
+
+def design_run(args):
+    """Bokulix and GPT-2 side by side at each of the named sizes: a prefill of 2,048 tokens (two prompts of 1,024) with its
+    share of the matrix peak, and decode steps at batch 1, 8 and 64 with their share of the HBM roofline."""
+    from liyab_amd.weights import write_random_model
+
+    short = "bf16" if args.dtype == "bfloat16" else "fp32"
+    runs = []
+    for size in args.design_sizes.split(","):
+        gpt2 = dict(SMALL, **SIZES[size])
+        if args.layers:
+            gpt2["n_layer"] = args.layers
+        designs = {"gpt2": gpt2, "bokulix": bokulix_config(gpt2, BOKULIX_SHAPES[size])}
+        ctx = gpt2["n_positions"]
+        k = max(16, min(args.steps, 128, ctx - args.prompt - 16))
+        for name, cfg in designs.items():
+            with tempfile.TemporaryDirectory() as d:
+                write_random_model(d, cfg, WEIGHT_SEEDS[size], dtype="bfloat16" if short == "bf16" else "float32")
+                engine = make_engine(d, args.dtype, 64, ctx, page_size=args.page_size, phases=args.phases)
+                lens = [1024, 1024]
+                ptps, pms = prefill_run(engine, cfg, lens)
+                flops = bokulix_prefill_flops(cfg, lens, 2) if name == "bokulix" else prefill_flops(cfg, lens, 2)
+                run = {"design": name, "size": size, "layers": gpt2["n_layer"],
+                       "prefill": {"tokens": 2048, "tok_s": round(ptps, 1), "ms": round(pms, 4), "gflop": round(flops / 1e9, 1),
+                                   "frac_of_matrix_peak": round(flops / (pms * 1e-3) / MFMA_PEAK[short], 4)}}
+                if args.phases:
+                    run["prefill"]["phases_ms"] = {n: round(v / 7, 4) for n, v in engine.phases_ms(reset=True).items()}  # (prefill_run steps 7 times)
+                for b in (1, 8, 64):
+                    bytes_fn = bokulix_step_bytes(cfg, b) if name == "bokulix" else None
+                    t, ms, nbytes = decode_run(engine, cfg, b, args.prompt, k, 4, step_bytes=bytes_fn)
+                    run[f"decode_b{b}"] = {"tok_s": round(t, 1), "ms_per_step": round(ms, 4), "mbytes_per_step": round(nbytes / 1e6, 1),
+                                           "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+                    if args.phases:
+                        # the run's prompts went through the same timer: the same prompts alone are taken off
+                        whole = engine.phases_ms(reset=True)
+                        decode_run(engine, cfg, b, args.prompt, 0, 0, step_bytes=bytes_fn)
+                        prompts = engine.phases_ms(reset=True)
+                        run[f"decode_b{b}"]["phases_ms"] = {n: round(max(v - prompts.get(n, 0.0), 0.0) / (k + 4), 4) for n, v in whole.items()}
+                runs.append(run)
+                del engine
+    print(json.dumps({"metric": "Bokulix beside GPT-2 at equal layer sizes: prefill of 2,048 tokens and decode steps", "dtype": short,
+                      "data": "synthetic", "page_size": args.page_size, "prompt_len": args.prompt, "runs": runs}))
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -367,6 +474,9 @@ def main():
     ap.add_argument("--link-floor", action="store_true", help="measure what one dependent kernel of a replayed graph costs at least")
     ap.add_argument("--phases", action="store_true", help="device milliseconds per phase of the forward pass (embed, attention, dense_ffn, lm_head) a decode step "
                     "and a prefill of 2,048 tokens, as the reference's command line prints them (tools/liyab_cli.cpp:198-211); steps run kernel by kernel, without graphs")
+    ap.add_argument("--design", default="", choices=["", "bokulix"],
+                    help="bokulix: that design beside GPT-2 at equal layer sizes (prefill and decode, both with their rooflines)")
+    ap.add_argument("--design-sizes", default="small,medium,xl", help="the sizes --design runs (of small, medium, xl)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -382,6 +492,8 @@ def main():
     if args.link_floor:
         print(json.dumps(link_floor()))
         return 0
+    if args.design:
+        return design_run(args)
     if args.workload:
         args.size = "medium" if args.workload == "medium16" else "xl"
     cfg = dict(SMALL, **SIZES[args.size])
