@@ -21,7 +21,8 @@
 
 namespace liyab {
 
-constexpr int kGroupedRows = 64;  // rows a tile; liyab_moe_align lays its lists out in these
+constexpr int kGroupedRows = 64;  // rows a tile; liyab_moe_align lays its lists out in these,
+constexpr int kSkinnyRows = 16;   // or in these for steps whose experts get few rows each
 
 struct GroupedParams {
     const void* a;
@@ -39,6 +40,7 @@ struct GroupedParams {
     int64_t gate_stride;
     int gate_dtype;
     int M, N, K;
+    int block;  // places a tile of rows_list: kGroupedRows, or kSkinnyRows for steps of few rows
 };
 
 __device__ __forceinline__ float gp_sigmoid(float z) { return 1.0f / (1.0f + expf(-z)); }
@@ -66,7 +68,7 @@ __device__ __forceinline__ int grouped_rows(const GroupedParams& p, int* idx) {
     if (p.rows_list != nullptr) {
         g = p.tile_group[tile];
         if (g < 0) return -1;
-        for (int i = threadIdx.x; i < kGroupedRows; i += blockDim.x) idx[i] = p.rows_list[tile * kGroupedRows + i];
+        for (int i = threadIdx.x; i < kGroupedRows; i += blockDim.x) idx[i] = i < p.block ? p.rows_list[tile * p.block + i] : -1;
     } else {
         g = blockIdx.z;
         for (int i = threadIdx.x; i < kGroupedRows; i += blockDim.x) {
@@ -106,44 +108,67 @@ grouped_mfma_kernel(GroupedParams p) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[u][r] = 0.0f;
 
-    // a thread's two 16-byte pieces of each operand tile: rows tid / 8 and tid / 8 + 32, k piece tid % 8
+    // a thread's two 16-byte pieces of each operand tile: rows tid / 8 and tid / 8 + 32, k piece tid % 8.
+    // Every load is made, from a row that exists (an empty place reads the first row, a feature past N the
+    // first feature, a piece past K the row's last piece) and masked afterwards: a load under a branch is
+    // waited for where the branch ends, and the pieces of kStages tiles of K are to be in flight together.
     const int row_a = tid / 8, kc = (tid % 8) * 8;
     const bf16_t* a_src[2];
     const bf16_t* w_src[NW][2];
+    bool a_ok[2], w_ok[2];
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
         const int id = idx[row_a + 32 * i];
-        a_src[i] = id >= 0 ? a + static_cast<int64_t>(id / p.a_div) * p.lda : nullptr;
+        a_ok[i] = id >= 0;
+        a_src[i] = a + static_cast<int64_t>(a_ok[i] ? id / p.a_div : 0) * p.lda;
         const int n = n0 + row_a + 32 * i;
+        w_ok[i] = n < N;
 #pragma unroll
-        for (int u = 0; u < NW; ++u) w_src[u][i] = n < N ? w[u] + static_cast<int64_t>(n) * K : nullptr;
+        for (int u = 0; u < NW; ++u) w_src[u][i] = w[u] + static_cast<int64_t>(w_ok[i] ? n : 0) * K;
     }
     const gp_u32x4 zero = {0, 0, 0, 0};
-    for (int k0 = 0; k0 < K; k0 += GPK) {
-        gp_u32x4 ra[2], rw[NW][2];
+    constexpr int kStages = 4;  // tiles of K whose pieces are in flight: a tile's trip from memory is most of its time otherwise
+    gp_u32x4 ra[kStages][2], rw[kStages][NW][2];
+    auto fetch = [&](int s, int k0) {
+        const int k = min(k0 + kc, K - 8);
         const bool in_k = k0 + kc < K;
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
-            ra[i] = (a_src[i] != nullptr && in_k) ? *reinterpret_cast<const gp_u32x4*>(a_src[i] + k0 + kc) : zero;
-#pragma unroll
-            for (int u = 0; u < NW; ++u) rw[u][i] = (w_src[u][i] != nullptr && in_k) ? *reinterpret_cast<const gp_u32x4*>(w_src[u][i] + k0 + kc) : zero;
-        }
-        __syncthreads();  // the previous tile's fragments have been read
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            *reinterpret_cast<gp_u32x4*>(lds + (row_a + 32 * i) * GPLD + kc) = ra[i];
-#pragma unroll
-            for (int u = 0; u < NW; ++u) *reinterpret_cast<gp_u32x4*>(lds + ((1 + u) * 64 + row_a + 32 * i) * GPLD + kc) = rw[u][i];
-        }
-        __syncthreads();
-        const bf16_t* Ab = lds + (wm * 32 + li) * GPLD + lk;
-#pragma unroll
-        for (int ks = 0; ks < GPK; ks += 16) {
-            const gp_bf16x8 fa = *reinterpret_cast<const gp_bf16x8*>(Ab + ks);
+            const gp_u32x4 va = *reinterpret_cast<const gp_u32x4*>(a_src[i] + k);
+            ra[s][i] = (a_ok[i] && in_k) ? va : zero;
 #pragma unroll
             for (int u = 0; u < NW; ++u) {
-                const gp_bf16x8 fw = *reinterpret_cast<const gp_bf16x8*>(lds + ((1 + u) * 64 + wn * 32 + li) * GPLD + lk + ks);
-                acc[u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fw, acc[u], 0, 0, 0);
+                const gp_u32x4 vw = *reinterpret_cast<const gp_u32x4*>(w_src[u][i] + k);
+                rw[s][u][i] = (w_ok[i] && in_k) ? vw : zero;
+            }
+        }
+    };
+    const int nk = (K + GPK - 1) / GPK;
+#pragma unroll
+    for (int s = 0; s < kStages; ++s) fetch(s, min(s, nk - 1) * GPK);  // (a stage past the last tile reads the last one again, unused)
+    for (int kb = 0; kb < nk; kb += kStages) {
+#pragma unroll
+        for (int s = 0; s < kStages; ++s) {
+            if (kb + s < nk) {  // (the same for every thread of the workgroup)
+                lds_barrier();  // the previous tile's fragments have been read
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    *reinterpret_cast<gp_u32x4*>(lds + (row_a + 32 * i) * GPLD + kc) = ra[s][i];
+#pragma unroll
+                    for (int u = 0; u < NW; ++u) *reinterpret_cast<gp_u32x4*>(lds + ((1 + u) * 64 + row_a + 32 * i) * GPLD + kc) = rw[s][u][i];
+                }
+                fetch(s, min(kb + s + kStages, nk - 1) * GPK);
+                lds_barrier();
+                const bf16_t* Ab = lds + (wm * 32 + li) * GPLD + lk;
+#pragma unroll
+                for (int ks = 0; ks < GPK; ks += 16) {
+                    const gp_bf16x8 fa = *reinterpret_cast<const gp_bf16x8*>(Ab + ks);
+#pragma unroll
+                    for (int u = 0; u < NW; ++u) {
+                        const gp_bf16x8 fw = *reinterpret_cast<const gp_bf16x8*>(lds + ((1 + u) * 64 + wn * 32 + li) * GPLD + lk + ks);
+                        acc[u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fw, acc[u], 0, 0, 0);
+                    }
+                }
             }
         }
     }
@@ -155,6 +180,100 @@ grouped_mfma_kernel(GroupedParams p) {
         const int id = idx[wm * 32 + 4 * (lane / 32) + 8 * (r / 4) + r % 4];
         if (id >= 0) grouped_store<NW>(p, id, g, n, acc[0][r], NW == 2 ? acc[NW - 1][r] : 0.0f);
     }
+}
+
+// Few rows a group (decoding: an expert gets a token or two): the product is a stream of the group's
+// weights, and what matters is how many workgroups pull on it. A workgroup owns 16 output features and one
+// tile of 16 row places; its four waves deal the units of 64 k among themselves and add their sums through
+// LDS in wave order. With v_mfma_f32_16x16x32_bf16 the weights are the first operand and the rows the second,
+// both straight from global memory into registers, 16 bytes a lane, a trip ahead of the multiplies. The order
+// of an element's sum depends on K alone.
+typedef __attribute__((ext_vector_type(4))) float gp_floatx4;
+union GpFrag {
+    gp_u32x4 u;
+    gp_bf16x8 v;
+};
+
+template <int NW>
+__global__ void __launch_bounds__(256)
+grouped_skinny_kernel(GroupedParams p) {
+    __shared__ float red[4 * NW * 256];
+    const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+    const int i = lane % 16, q = lane / 16;
+    const int tile = blockIdx.x;
+    int g;
+    if (p.rows_list != nullptr) {
+        g = p.tile_group[tile];
+        if (g < 0) return;
+    } else {
+        g = blockIdx.z;
+    }
+    auto row_id = [&](int place) {
+        if (p.rows_list != nullptr) return p.rows_list[tile * kSkinnyRows + place];
+        const int m = tile * kSkinnyRows + place;
+        return m < p.M ? m : -1;
+    };
+    const int N = p.N, K = p.K, n0 = blockIdx.y * 16;
+    const int my_id = row_id(i);
+    // an empty place reads the first row, a feature past N the last one: computed, never stored
+    const bf16_t* arow = static_cast<const bf16_t*>(p.a) + static_cast<int64_t>(my_id >= 0 ? my_id / p.a_div : 0) * p.lda + static_cast<int64_t>(g) * p.a_group_cols;
+    const int64_t wrow = (static_cast<int64_t>(g) * N + min(n0 + i, N - 1)) * K;
+    const bf16_t* w[2] = {static_cast<const bf16_t*>(p.w0) + wrow, NW == 2 ? static_cast<const bf16_t*>(p.w1) + wrow : nullptr};
+    const gp_u32x4 zero = {0, 0, 0, 0};
+    // a lane's two pieces of a unit of 64 k: k0 + 8 q and k0 + 32 + 8 q; a piece past K reads the row's last piece, as zeros for the weights
+    auto fetch = [&](int unit, GpFrag (&x)[2], GpFrag (&wf)[NW][2]) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int k = unit * 64 + 32 * h + 8 * q;
+            const int kk = min(k, K - 8);
+            x[h].u = *reinterpret_cast<const gp_u32x4*>(arow + kk);
+#pragma unroll
+            for (int u = 0; u < NW; ++u) {
+                const gp_u32x4 v = *reinterpret_cast<const gp_u32x4*>(w[u] + kk);
+                wf[u][h].u = k < K ? v : zero;
+            }
+        }
+    };
+    gp_floatx4 acc[NW];
+#pragma unroll
+    for (int u = 0; u < NW; ++u) acc[u] = gp_floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    const int units = (K + 63) / 64;
+    GpFrag xc[2], wc[NW][2];
+    int unit = wave;
+    if (unit < units) fetch(unit, xc, wc);
+    while (unit < units) {  // (the same trips for every lane of a wave)
+        const int next = unit + 4;
+        GpFrag xn[2], wn[NW][2];
+        if (next < units) fetch(next, xn, wn);
+#pragma unroll
+        for (int u = 0; u < NW; ++u) {
+            acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[u][0].v, xc[0].v, acc[u], 0, 0, 0);
+            acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[u][1].v, xc[1].v, acc[u], 0, 0, 0);
+        }
+        if (next < units) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                xc[h] = xn[h];
+#pragma unroll
+                for (int u = 0; u < NW; ++u) wc[u][h] = wn[u][h];
+            }
+        }
+        unit = next;
+    }
+    // acc[u][r] = this wave's share of C^T[n = 4 q + r][m = i]; kept [wave][matrix][m][n]
+#pragma unroll
+    for (int u = 0; u < NW; ++u)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) red[(wave * NW + u) * 256 + i * 16 + 4 * q + r] = acc[u][r];
+    __syncthreads();
+    const int m = tid / 16, n = n0 + tid % 16;
+    float v[2] = {0.0f, 0.0f};
+#pragma unroll
+    for (int u = 0; u < NW; ++u)
+#pragma unroll
+        for (int wv = 0; wv < 4; ++wv) v[u] += red[(wv * NW + u) * 256 + tid];
+    const int id = row_id(m);
+    if (id >= 0 && n < N) grouped_store<NW>(p, id, g, n, v[0], v[1]);
 }
 
 // Plain 32-bit multiply-adds: a tile of 64 rows x 64 output features, a thread 4 x 4 of them, K in
@@ -229,26 +348,33 @@ using namespace liyab;
 
 // See the head of this file. dtype: the element type of a, w0 and w1. n_groups: heads (rows_list
 // null) or experts (the values of tile_group lie below it; the caller has made them so). n_tiles:
-// the tiles of rows to launch (with rows_list: the length of tile_group; without: (M + 63) / 64).
+// the tiles of rows to launch (with rows_list: the length of tile_group; without: (M + block - 1) / block).
+// block: the row places a tile, 64, or 16 for steps of few rows a group (bfloat16 operands in 16-byte pieces).
 extern "C" int liyab_grouped_product(const void* a, int64_t lda, int a_div, int a_group_cols, const void* w0, const void* w1, int dtype,
                                      void* out, int out_dtype, int64_t ldo, int out_group_cols, const int* rows_list,
-                                     const int* tile_group, int n_tiles, int n_groups, const float* row_scale, const void* gate,
-                                     int gate_dtype, int64_t gate_stride, int M, int N, int K, hipStream_t stream) {
+                                     const int* tile_group, int n_tiles, int block, int n_groups, const float* row_scale,
+                                     const void* gate, int gate_dtype, int64_t gate_stride, int M, int N, int K, hipStream_t stream) {
     LIYAB_REQUIRE(a && w0 && out, "grouped_product: null pointer");
     LIYAB_REQUIRE(dtype == kF32 || dtype == kBF16, "grouped_product: unknown dtype %d", dtype);
     LIYAB_REQUIRE(out_dtype == kF32 || out_dtype == kBF16, "grouped_product: unknown output dtype %d", out_dtype);
     LIYAB_REQUIRE(M >= 0 && N > 0 && K > 0 && a_div >= 1 && n_groups >= 1 && n_groups <= 65535 && n_tiles >= 0, "grouped_product: bad sizes M=%d N=%d K=%d", M, N, K);
     LIYAB_REQUIRE((rows_list == nullptr) == (tile_group == nullptr), "grouped_product: a list of rows goes with the groups of its tiles");
-    LIYAB_REQUIRE(rows_list != nullptr || n_tiles == (M + kGroupedRows - 1) / kGroupedRows, "grouped_product: %d tiles for %d rows", n_tiles, M);
+    LIYAB_REQUIRE(block == kGroupedRows || block == kSkinnyRows, "grouped_product: tiles of %d rows (%d or %d)", block, kGroupedRows, kSkinnyRows);
+    LIYAB_REQUIRE(rows_list != nullptr || n_tiles == (M + block - 1) / block, "grouped_product: %d tiles for %d rows", n_tiles, M);
     LIYAB_REQUIRE(gate == nullptr || gate_dtype == kF32 || gate_dtype == kBF16, "grouped_product: unknown gate dtype %d", gate_dtype);
     LIYAB_REQUIRE(gate == nullptr || gate_stride >= static_cast<int64_t>(rows_list ? 1 : n_groups) * N, "grouped_product: the gate's rows are shorter than the output's");
     if (M == 0 || n_tiles == 0) return 0;
-    GroupedParams p{a, lda, a_div, a_group_cols, w0, w1, out, ldo, out_group_cols, out_dtype, rows_list, tile_group, row_scale, gate, gate_stride, gate_dtype, M, N, K};
+    GroupedParams p{a, lda, a_div, a_group_cols, w0, w1, out, ldo, out_group_cols, out_dtype, rows_list, tile_group, row_scale, gate, gate_stride, gate_dtype, M, N, K, block};
     const dim3 grid(n_tiles, (N + 63) / 64, rows_list ? 1 : n_groups);
     const bool matrix = dtype == kBF16 && K % 8 == 0 && lda % 8 == 0 && a_group_cols % 8 == 0 &&
                         (reinterpret_cast<uintptr_t>(a) & 15) == 0 && (reinterpret_cast<uintptr_t>(w0) & 15) == 0 &&
                         (reinterpret_cast<uintptr_t>(w1) & 15) == 0;
-    if (matrix) {
+    LIYAB_REQUIRE(block == kGroupedRows || matrix, "grouped_product: tiles of %d rows are for bfloat16 operands in 16-byte pieces", kSkinnyRows);
+    if (block == kSkinnyRows) {
+        const dim3 skinny(n_tiles, (N + 15) / 16, rows_list ? 1 : n_groups);
+        if (w1 != nullptr) grouped_skinny_kernel<2><<<skinny, 256, 0, stream>>>(p);
+        else grouped_skinny_kernel<1><<<skinny, 256, 0, stream>>>(p);
+    } else if (matrix) {
         if (w1 != nullptr) grouped_mfma_kernel<2><<<grid, 256, 0, stream>>>(p);
         else grouped_mfma_kernel<1><<<grid, 256, 0, stream>>>(p);
     } else if (dtype == kBF16) {

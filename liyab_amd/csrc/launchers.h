@@ -71,9 +71,11 @@ int liyab_latent_store(void* cache, int dtype, const void* src, int64_t src_stri
                        const int* slots, int n, int rank, int page_size, int num_pages, hipStream_t stream);
 int liyab_grouped_product(const void* a, int64_t lda, int a_div, int a_group_cols, const void* w0, const void* w1, int dtype, void* out,
                           int out_dtype, int64_t ldo, int out_group_cols, const int* rows_list, const int* tile_group, int n_tiles,
-                          int n_groups, const float* row_scale, const void* gate, int gate_dtype, int64_t gate_stride, int M, int N,
+                          int block, int n_groups, const float* row_scale, const void* gate, int gate_dtype, int64_t gate_stride, int M, int N,
                           int K, hipStream_t stream);
 int liyab_moe_route(const float* logits, int64_t ld, int n, int n_experts, int top, int* ids, float* weights, hipStream_t stream);
+int liyab_moe_route_align(const float* logits, int64_t ld, int n, int n_experts, int top, int* ids, float* weights, int block,
+                          int* rows_list, int* tile_group, int max_tiles, hipStream_t stream);
 int liyab_moe_align(const int* ids, int n_entries, int n_experts, int block, int* rows_list, int* tile_group, int max_tiles,
                     hipStream_t stream);
 

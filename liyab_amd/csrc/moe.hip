@@ -10,6 +10,8 @@
 // tile_group [max_tiles] (the expert of each tile, -1 for a tile that is not used). max_tiles is
 // a bound that the step's sizes fix (entries / block + min(experts, entries), rounded up), so
 // that the products' grids do not depend on where the tokens went. One workgroup.
+//
+// liyab_moe_route_align: both in one launch, for steps of at most 1,024 tokens.
 #include "common.h"
 #include "launchers.h"
 
@@ -17,11 +19,8 @@ namespace liyab {
 
 constexpr int kMaxTop = 32;
 
-__global__ void __launch_bounds__(256)
-moe_route_kernel(const float* __restrict__ logits, int64_t ld, int n, int E, int top, int* __restrict__ ids, float* __restrict__ weights) {
-    const int t = blockIdx.x * 256 + threadIdx.x;
-    if (t >= n) return;
-    const float* z = logits + static_cast<int64_t>(t) * ld;
+// One token's choice: the `top` largest of its E logits (the lower number among equals) and the softmax over them.
+__device__ __forceinline__ void route_token(const float* __restrict__ z, int E, int top, int* __restrict__ ids, float* __restrict__ weights) {
     int chosen[kMaxTop];
     float value[kMaxTop];
     for (int k = 0; k < top; ++k) {
@@ -46,17 +45,23 @@ moe_route_kernel(const float* __restrict__ logits, int64_t ld, int n, int E, int
         sum += value[k];
     }
     for (int k = 0; k < top; ++k) {
-        ids[static_cast<int64_t>(t) * top + k] = chosen[k];
-        weights[static_cast<int64_t>(t) * top + k] = value[k] / sum;
+        ids[k] = chosen[k];
+        weights[k] = value[k] / sum;
     }
 }
 
-__global__ void __launch_bounds__(1024)
-moe_align_kernel(const int* __restrict__ ids, int n_entries, int E, int block, int* __restrict__ rows_list, int* __restrict__ tile_group,
-                 int max_tiles) {
-    extern __shared__ int sh[];  // counts [E], first place of each expert [E + 1]
-    int* counts = sh;
-    int* first = sh + E;
+__global__ void __launch_bounds__(256)
+moe_route_kernel(const float* __restrict__ logits, int64_t ld, int n, int E, int top, int* __restrict__ ids, float* __restrict__ weights) {
+    const int t = blockIdx.x * 256 + threadIdx.x;
+    if (t >= n) return;
+    route_token(logits + static_cast<int64_t>(t) * ld, E, top, ids + static_cast<int64_t>(t) * top, weights + static_cast<int64_t>(t) * top);
+}
+
+// The entries of `ids` listed by expert in tiles of `block` places; one workgroup of 1,024 threads runs this.
+__device__ __forceinline__ void align_entries(const int* __restrict__ ids, int n_entries, int E, int block, int* __restrict__ rows_list,
+                                              int* __restrict__ tile_group, int max_tiles, int* sh) {
+    int* counts = sh;     // [E]
+    int* first = sh + E;  // [E + 1]: the first place of each expert
     const int tid = threadIdx.x;
     for (int e = tid; e < E; e += 1024) counts[e] = 0;
     for (int i = tid; i < max_tiles * block; i += 1024) rows_list[i] = -1;
@@ -88,6 +93,24 @@ moe_align_kernel(const int* __restrict__ ids, int n_entries, int E, int block, i
     }
 }
 
+__global__ void __launch_bounds__(1024)
+moe_align_kernel(const int* __restrict__ ids, int n_entries, int E, int block, int* __restrict__ rows_list, int* __restrict__ tile_group,
+                 int max_tiles) {
+    extern __shared__ int sh[];
+    align_entries(ids, n_entries, E, block, rows_list, tile_group, max_tiles, sh);
+}
+
+// Both in one launch for steps of at most 1,024 tokens: a thread routes a token, then the workgroup lists the entries.
+__global__ void __launch_bounds__(1024)
+moe_route_align_kernel(const float* __restrict__ logits, int64_t ld, int n, int E, int top, int* __restrict__ ids, float* __restrict__ weights,
+                       int block, int* __restrict__ rows_list, int* __restrict__ tile_group, int max_tiles) {
+    extern __shared__ int sh[];
+    const int t = threadIdx.x;
+    if (t < n) route_token(logits + static_cast<int64_t>(t) * ld, E, top, ids + static_cast<int64_t>(t) * top, weights + static_cast<int64_t>(t) * top);
+    __syncthreads();  // (the ids are read back by other threads of this workgroup)
+    align_entries(ids, n * top, E, block, rows_list, tile_group, max_tiles, sh);
+}
+
 }  // namespace liyab
 
 using namespace liyab;
@@ -110,4 +133,17 @@ extern "C" int liyab_moe_align(const int* ids, int n_entries, int n_experts, int
     if (n_entries == 0) return 0;
     moe_align_kernel<<<1, 1024, (2 * n_experts + 1) * sizeof(int), stream>>>(ids, n_entries, n_experts, block, rows_list, tile_group, max_tiles);
     return check_launch("moe_align");
+}
+
+extern "C" int liyab_moe_route_align(const float* logits, int64_t ld, int n, int n_experts, int top, int* ids, float* weights, int block,
+                                     int* rows_list, int* tile_group, int max_tiles, hipStream_t stream) {
+    LIYAB_REQUIRE(n <= 1024, "moe_route_align: %d tokens; one workgroup routes at most 1,024 (moe_route and moe_align take more)", n);
+    if (const int rc = liyab_moe_route(logits, ld, 0, n_experts, top, ids, weights, stream)) return rc;                    // (the checks of both,
+    if (const int rc = liyab_moe_align(ids, 0, n_experts, block, rows_list, tile_group, max_tiles, stream)) return rc;    //  nothing launched)
+    LIYAB_REQUIRE(n >= 0 && static_cast<int64_t>(max_tiles) * block >= static_cast<int64_t>(n) * top + static_cast<int64_t>(n * top < n_experts ? n * top : n_experts) * (block - 1),
+                  "moe_route_align: %d tiles of %d places do not hold %d entries of %d experts", max_tiles, block, n * top, n_experts);
+    if (n == 0) return 0;
+    moe_route_align_kernel<<<1, 1024, (2 * n_experts + 1) * sizeof(int), stream>>>(logits, ld, n, n_experts, top, ids, weights, block, rows_list,
+                                                                                    tile_group, max_tiles);
+    return check_launch("moe_route_align");
 }

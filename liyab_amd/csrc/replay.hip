@@ -95,6 +95,7 @@ static const Entry kEntries[] = {
     LIYAB_ENTRY(liyab_grouped_product),
     LIYAB_ENTRY(liyab_moe_route),
     LIYAB_ENTRY(liyab_moe_align),
+    LIYAB_ENTRY(liyab_moe_route_align),
 };
 constexpr int kNumEntries = static_cast<int>(sizeof(kEntries) / sizeof(kEntries[0]));
 

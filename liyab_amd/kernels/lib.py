@@ -77,10 +77,11 @@ _SIGNATURES = {
     "liyab_causal_conv": [P, P, c_int, P, P, c_int, P, c_int, P, P, P, P, c_int, c_int, P],
     "liyab_keep_rows": [P, c_int, c_int, P, P, P, P, P, P, c_int, c_int, P],
     "liyab_latent_store": [P, c_int, P, c_int64, c_int, P, c_float, P, c_int, c_int, c_int, c_int, P],
-    "liyab_grouped_product": [P, c_int64, c_int, c_int, P, P, c_int, P, c_int, c_int64, c_int, P, P, c_int, c_int, P, P, c_int, c_int64,
+    "liyab_grouped_product": [P, c_int64, c_int, c_int, P, P, c_int, P, c_int, c_int64, c_int, P, P, c_int, c_int, c_int, P, P, c_int, c_int64,
                               c_int, c_int, c_int, P],
     "liyab_moe_route": [P, c_int64, c_int, c_int, c_int, P, P, P],
     "liyab_moe_align": [P, c_int, c_int, c_int, P, P, c_int, P],
+    "liyab_moe_route_align": [P, c_int64, c_int, c_int, c_int, P, P, c_int, P, P, c_int, P],
 }
 
 

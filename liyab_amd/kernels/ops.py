@@ -1134,6 +1134,7 @@ def latent_store(cache: torch.Tensor, src: torch.Tensor, col_off: int, weight: O
 
 
 GROUPED_ROWS = 64  # rows a tile of the grouped product (csrc/grouped_product.hip: kGroupedRows)
+SKINNY_ROWS = 16  # or as few as this, for steps in which a group gets few rows (kSkinnyRows)
 
 
 def heads_product(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, gate: Optional[torch.Tensor] = None) -> None:
@@ -1154,47 +1155,64 @@ def heads_product(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, gate: Opt
         if tuple(gate.shape) != (n, H * N):
             raise KernelError(f"heads_product: the gate must be [{n}, {H * N}]")
     _lib.call("liyab_grouped_product", a.data_ptr(), lda, 1, K, w.data_ptr(), None, dtype_code(a.dtype), out.data_ptr(),
-              dtype_code(out.dtype), ldo, N, None, None, (n + GROUPED_ROWS - 1) // GROUPED_ROWS, H, None, _ptr(gate),
+              dtype_code(out.dtype), ldo, N, None, None, (n + GROUPED_ROWS - 1) // GROUPED_ROWS, GROUPED_ROWS, H, None, _ptr(gate),
               dtype_code(gate.dtype) if gate is not None else F32, gs, n, N, K, _stream())
 
 
 MOE_MAX_TOP = 32
 
 
-def moe_tiles(n_entries: int, n_experts: int) -> int:
-    """The tiles of GROUPED_ROWS places that hold `n_entries` entries listed by expert, whatever their
+def moe_tiles(n_entries: int, n_experts: int, block: int = GROUPED_ROWS) -> int:
+    """The tiles of `block` places that hold `n_entries` entries listed by expert, whatever their
     experts: a bound that follows from the sizes alone."""
-    return -(-(n_entries + min(n_entries, n_experts) * (GROUPED_ROWS - 1)) // GROUPED_ROWS)
+    return -(-(n_entries + min(n_entries, n_experts) * (block - 1)) // block)
+
+
+def moe_block(n_entries: int, n_experts: int, dtype: torch.dtype, *inner_sizes: int) -> int:
+    """The row places a tile for a step of `n_entries` (token, choice) entries: 16 while an expert gets 32
+    rows or fewer on average (the products are then streams of the chosen experts' weights, and tiles of 16
+    rows x 16 features make some hundred workgroups pull on them where tiles of 64 x 64 make a few dozen:
+    one token of 2 x 1,536 features over 768, 16.4 -> 6 us), 64 beyond; the small tiles are for bfloat16
+    operands whose inner sizes are multiples of 8."""
+    few = n_entries <= 32 * n_experts and dtype == torch.bfloat16 and all(k % 8 == 0 for k in inner_sizes)
+    return SKINNY_ROWS if few else GROUPED_ROWS
 
 
 def moe_route(logits: torch.Tensor, top: int, ids: torch.Tensor, weights: torch.Tensor, rows_list: torch.Tensor,
-              tile_group: torch.Tensor) -> None:
+              tile_group: torch.Tensor, block: int = GROUPED_ROWS) -> None:
     """From float32 router logits [n, experts] (rows may be strided): ids int32 and weights float32 [n,
     top] (the experts with the largest logits, softmax over those alone), and the entries t * top + k
-    listed by expert in tiles: rows_list int32 [tiles * GROUPED_ROWS] (-1: empty), tile_group int32
-    [tiles] (-1: unused), tiles = moe_tiles(n * top, experts)."""
+    listed by expert in tiles of `block` places: rows_list int32 [tiles * block] (-1: empty), tile_group
+    int32 [tiles] (-1: unused), tiles = moe_tiles(n * top, experts, block)."""
     ld = _rows(logits, "logits")
     n, E = logits.shape
     if logits.dtype != torch.float32:
         raise KernelError("moe_route: the logits must be float32")
     if not 1 <= top <= min(E, MOE_MAX_TOP):
         raise KernelError(f"moe_route: {top} of {E} experts a token (at most {MOE_MAX_TOP})")
-    tiles = moe_tiles(n * top, E)
+    if block not in (GROUPED_ROWS, SKINNY_ROWS):
+        raise KernelError(f"moe_route: tiles of {block} places ({GROUPED_ROWS} or {SKINNY_ROWS})")
+    tiles = moe_tiles(n * top, E, block)
     _i32(ids, "ids", n * top)
-    _i32(rows_list, "rows_list", tiles * GROUPED_ROWS)
+    _i32(rows_list, "rows_list", tiles * block)
     _i32(tile_group, "tile_group", tiles)
     _dev(weights, "weights")
     if weights.dtype != torch.float32 or weights.numel() < n * top or not weights.is_contiguous():
         raise KernelError("moe_route: weights must be contiguous float32 [n, top]")
+    if n <= 1024:  # one launch: a thread routes a token, then the workgroup lists the entries
+        _lib.call("liyab_moe_route_align", logits.data_ptr(), ld, n, E, top, ids.data_ptr(), weights.data_ptr(), block,
+                  rows_list.data_ptr(), tile_group.data_ptr(), tiles, _stream())
+        return
     _lib.call("liyab_moe_route", logits.data_ptr(), ld, n, E, top, ids.data_ptr(), weights.data_ptr(), _stream())
-    _lib.call("liyab_moe_align", ids.data_ptr(), n * top, E, GROUPED_ROWS, rows_list.data_ptr(), tile_group.data_ptr(), tiles, _stream())
+    _lib.call("liyab_moe_align", ids.data_ptr(), n * top, E, block, rows_list.data_ptr(), tile_group.data_ptr(), tiles, _stream())
 
 
 def moe_product(out: torch.Tensor, a: torch.Tensor, w0: torch.Tensor, w1: Optional[torch.Tensor], rows_list: torch.Tensor,
-                tile_group: torch.Tensor, *, a_div: int = 1, row_scale: Optional[torch.Tensor] = None) -> None:
+                tile_group: torch.Tensor, *, a_div: int = 1, row_scale: Optional[torch.Tensor] = None, block: int = GROUPED_ROWS) -> None:
     """For every listed entry e of expert g: out[e] = f(a[e // a_div] . w0[g]^T, a[e // a_div] . w1[g]^T) *
     row_scale[e], f(u, v) = silu(u) * v with two matrices and u with one. a [*, K] and out [entries, N]
-    contiguous, w0 / w1 [experts, N, K] in a's dtype; rows_list and tile_group as `moe_route` leaves them."""
+    contiguous, w0 / w1 [experts, N, K] in a's dtype; rows_list and tile_group as `moe_route` leaves them for
+    tiles of `block` places."""
     _dev(w0, "w0")
     if w0.dim() != 3 or not w0.is_contiguous() or w0.dtype != a.dtype:
         raise KernelError(f"moe_product: w0 must be contiguous [experts, N, K] in a's dtype, got {tuple(w0.shape)} {w0.dtype}")
@@ -1206,14 +1224,16 @@ def moe_product(out: torch.Tensor, a: torch.Tensor, w0: torch.Tensor, w1: Option
     if a.shape[1] != K or out.shape[1] != N or a_div < 1 or a.shape[0] * a_div < entries:
         raise KernelError(f"moe_product: a {tuple(a.shape)} / out {tuple(out.shape)} do not fit [{E}, {N}, {K}] with {a_div} entries a row")
     tiles = tile_group.numel()
-    if tiles < moe_tiles(entries, E):
+    if block not in (GROUPED_ROWS, SKINNY_ROWS) or (block == SKINNY_ROWS and (a.dtype != torch.bfloat16 or K % 8 != 0 or lda % 8 != 0)):
+        raise KernelError(f"moe_product: tiles of {block} places do not go with these operands")
+    if tiles < moe_tiles(entries, E, block):
         raise KernelError(f"moe_product: {tiles} tiles do not hold {entries} entries of {E} experts")
-    _i32(rows_list, "rows_list", tiles * GROUPED_ROWS)
+    _i32(rows_list, "rows_list", tiles * block)
     _i32(tile_group, "tile_group", tiles)
     if row_scale is not None:
         _dev(row_scale, "row_scale")
         if row_scale.dtype != torch.float32 or row_scale.numel() < entries or not row_scale.is_contiguous():
             raise KernelError("moe_product: row_scale must be contiguous float32 [entries]")
     _lib.call("liyab_grouped_product", a.data_ptr(), lda, a_div, 0, w0.data_ptr(), _ptr(w1), dtype_code(a.dtype), out.data_ptr(),
-              dtype_code(out.dtype), ldo, 0, rows_list.data_ptr(), tile_group.data_ptr(), tiles, E, _ptr(row_scale), None, F32, 0,
+              dtype_code(out.dtype), ldo, 0, rows_list.data_ptr(), tile_group.data_ptr(), tiles, block, E, _ptr(row_scale), None, F32, 0,
               entries, N, K, _stream())

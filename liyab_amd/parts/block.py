@@ -6,6 +6,7 @@ import torch
 
 from ..kernels import ops
 from .base import SplitStream, StepContext, settled
+from .linear import linear
 from .registry import register_block
 
 
@@ -101,6 +102,22 @@ class PostNormGatedBlock:
                 raise ValueError("a post-norm block's row update applies a root-mean-square norm (kind 'rmsnorm')")
         if mixer.state_spec() is not None and self.conv is not None and self.conv.state_spec() is not None:
             raise ValueError("a mixer with state of its own under an input convolution: one state a layer")
+        # The feed-forward's gate and its router read the same rows: one product [gate | router] instead of two
+        # (a launch less a layer). The joint matrix is made once for the two matrices it is made of, so that
+        # layers sharing their tensors share it, and the parts give theirs up.
+        self.joint_weight = self.joint_bias = None
+        if self.gate_ffn is not None and hasattr(ffn, "take_router") and ffn.router is not None and ffn.router.dtype == self.gate_ffn.weight.dtype:
+            gw, gb = self.gate_ffn.weight, self.gate_ffn.bias
+            rw, rb = ffn.take_router()
+            hit = getattr(gw, "_joint_rows", None)  # (layers that share their tensors get the same tensor objects from the store)
+            if hit is None or hit[2] is not rw:
+                bias = None
+                if gb is not None or rb is not None:
+                    bias = torch.cat([gb if gb is not None else torch.zeros(gw.shape[0], dtype=torch.float32, device=gw.device),
+                                      rb if rb is not None else torch.zeros(rw.shape[0], dtype=torch.float32, device=gw.device)])
+                hit = gw._joint_rows = (torch.cat([gw, rw], dim=0).contiguous(), bias, rw)
+            self.joint_weight, self.joint_bias = hit[0], hit[1]
+            self.gate_ffn.weight = self.gate_ffn.bias = None
 
     def state_spec(self):
         return (self.conv.state_spec() if self.conv is not None else None) or self.mixer.state_spec()
@@ -125,10 +142,16 @@ class PostNormGatedBlock:
         if self.ffn is not None:
             if ctx.phases is not None:
                 ctx.phases.mark(self.ffn_phase)
-            gate = self.gate_ffn.forward(xh, ctx, "gate_logits") if self.gate_ffn is not None else None
             k = int(getattr(self.ffn, "rows_a_token", 1))
             y = ws.get("sublayer_rows", (n * k, d), torch.float32) if k > 1 else y
-            self.ffn.forward(xh, ctx, None, out=y)
+            if self.joint_weight is not None:
+                z = ws.get("gate_router_logits", (n, self.joint_weight.shape[0]), torch.float32)
+                linear(xh, self.joint_weight, self.joint_bias, out=z)
+                gate = z[:, :d]
+                self.ffn.forward(xh, ctx, None, out=y, router_logits=z[:, d:])
+            else:
+                gate = self.gate_ffn.forward(xh, ctx, "gate_logits") if self.gate_ffn is not None else None
+                self.ffn.forward(xh, ctx, None, out=y)
             ops.gated_norm_add(x, y, self.norm_ffn.weight, self.norm_ffn.eps, n_sum=k, gate=gate)
         return None
 

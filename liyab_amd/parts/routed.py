@@ -37,25 +37,39 @@ class RoutedFFN:
         self.up = store.fetch_joined([t[("up", e)] for e in range(E)], [(F, d)] * E, "matrix", "stack")
         self.down = store.fetch_joined([t[("down", e)] for e in range(E)], [(d, F)] * E, "matrix", "stack")
 
+    def take_router(self):
+        """(weight [experts, width], bias or None): the router's product handed to a caller that runs it as rows
+        of a wider product over the same input and passes the logits to `forward(..., router_logits=)`; this
+        part then no longer holds the matrix."""
+        w, b = self.router, self.router_bias
+        self.router = self.router_bias = None
+        return w, b
+
     rows_a_token = property(lambda self: self.top)  # rows `forward(..., out=)` leaves for each token
 
-    def forward(self, h, ctx: StepContext, residual: Optional[torch.Tensor], out: Optional[torch.Tensor] = None):
+    def forward(self, h, ctx: StepContext, residual: Optional[torch.Tensor], out: Optional[torch.Tensor] = None,
+                router_logits: Optional[torch.Tensor] = None):
         """Adds the result into `residual`, or, with `out` (float32 [n * top, width]), leaves each token's
-        `top` weighted expert outputs there in consecutive rows, for a reader that adds them up."""
+        `top` weighted expert outputs there in consecutive rows, for a reader that adds them up.
+        `router_logits` (float32 [n, experts], rows may be strided): the router's logits where the caller
+        has computed them already, beside a product of its own over the same rows (`take_router`)."""
         h = as_tensor(h)
         n, ws, E, top = h.shape[0], ctx.workspace, self.n_experts, self.top
-        logits = ws.get("router_logits", (n, E), torch.float32)
-        linear(h, self.router, self.router_bias, out=logits)
-        tiles = ops.moe_tiles(n * top, E)
+        logits = router_logits
+        if logits is None:
+            logits = ws.get("router_logits", (n, E), torch.float32)
+            linear(h, self.router, self.router_bias, out=logits)
+        block = ops.moe_block(n * top, E, self.dtype, self.width, self.inner)
+        tiles = ops.moe_tiles(n * top, E, block)
         ids = ws.get("routed_ids", (n * top,), torch.int32)
         weights = ws.get("routed_weights", (n * top,), torch.float32)
-        rows_list = ws.get("routed_rows", (tiles * ops.GROUPED_ROWS,), torch.int32)
+        rows_list = ws.get("routed_rows", (tiles * block,), torch.int32)
         tile_group = ws.get("routed_tiles", (tiles,), torch.int32)
-        ops.moe_route(logits, top, ids, weights, rows_list, tile_group)
+        ops.moe_route(logits, top, ids, weights, rows_list, tile_group, block=block)
         inner = ws.get("routed_inner", (n * top, self.inner), self.dtype)
-        ops.moe_product(inner, h, self.gate, self.up, rows_list, tile_group, a_div=top)
+        ops.moe_product(inner, h, self.gate, self.up, rows_list, tile_group, a_div=top, block=block)
         y = out if out is not None else ws.get("routed_out", (n * top, self.width), torch.float32)
-        ops.moe_product(y, inner, self.down, None, rows_list, tile_group, row_scale=weights)
+        ops.moe_product(y, inner, self.down, None, rows_list, tile_group, row_scale=weights, block=block)
         if out is None:
             ops.gated_norm_add(settled(residual), y, None, 0.0, n_sum=top, normalize=False)
         return None

@@ -199,9 +199,10 @@ def test_products_a_head_alone(dtype, shape):
         assert tt.rel_err(f64(out32), want * plain.sigmoid(f64(glog))) < (1e-6 if dtype == "float32" else 1e-5)
 
 
+@pytest.mark.parametrize("block", [64, 16])
 @pytest.mark.parametrize("experts,top", [(8, 2), (3, 3), (5, 1), (64, 6)])
-@pytest.mark.parametrize("n", [1, 7, 300])
-def test_routing_alone(experts, top, n):
+@pytest.mark.parametrize("n", [1, 7, 300, 1500])
+def test_routing_alone(experts, top, n, block):
     """The chosen experts and their weights against the twin's; every (token, choice) entry stands exactly
     once in its expert's tiles, tiles no expert uses are marked, and equal logits go to the lower number."""
     from liyab_amd.kernels import ops
@@ -209,12 +210,12 @@ def test_routing_alone(experts, top, n):
     rng = np.random.default_rng(3)
     logits = rand(rng, n, experts + 5, scale=3.0).to(DEV)[:, 2:2 + experts]
     logits[0, :] = 0.25  # all equal: the first `top` experts
-    tiles = ops.moe_tiles(n * top, experts)
+    tiles = ops.moe_tiles(n * top, experts, block)
     ids = torch.empty(n * top, dtype=torch.int32, device=DEV)
     weights = torch.empty(n * top, dtype=torch.float32, device=DEV)
-    rows_list = torch.full((tiles * ops.GROUPED_ROWS,), -7, dtype=torch.int32, device=DEV)
+    rows_list = torch.full((tiles * block,), -7, dtype=torch.int32, device=DEV)
     tile_group = torch.full((tiles,), -7, dtype=torch.int32, device=DEV)
-    ops.moe_route(logits, top, ids, weights, rows_list, tile_group)
+    ops.moe_route(logits, top, ids, weights, rows_list, tile_group, block=block)
     z = f64(logits)
     order = np.argsort(-z, axis=-1, kind="stable")[:, :top]
     chosen = np.take_along_axis(z, order, -1)
@@ -235,13 +236,17 @@ def test_routing_alone(experts, top, n):
     assert sorted(seen) == list(range(n * top))
 
 
-@pytest.mark.parametrize("sizes", [(8, 2, 64, 96), (3, 3, 50, 100), (6, 1, 24, 40)])
+@pytest.mark.parametrize("block", [64, 16])
+@pytest.mark.parametrize("sizes", [(8, 2, 64, 96), (3, 3, 50, 100), (6, 1, 24, 40), (4, 2, 200, 136)])
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_routed_products_alone(dtype, sizes):
-    """The two grouped products over the routed entries against a loop over tokens and choices."""
+def test_routed_products_alone(dtype, sizes, block):
+    """The two grouped products over the routed entries against a loop over tokens and choices, in tiles of
+    64 row places and in the tiles of 16 that steps of few rows take."""
     from liyab_amd.kernels import ops
 
     E, top, F, d = sizes
+    if block == 16 and (dtype == "float32" or F % 8 or d % 8):
+        pytest.skip("tiles of 16 row places are for bfloat16 operands in 16-byte pieces")
     dt = torch.float32 if dtype == "float32" else torch.bfloat16
     rng = np.random.default_rng(4)
     for n in (1, 9, 150):
@@ -249,14 +254,14 @@ def test_routed_products_alone(dtype, sizes):
         wg, wu = rand(rng, E, F, d, scale=d ** -0.5).to(dt).to(DEV), rand(rng, E, F, d, scale=d ** -0.5).to(dt).to(DEV)
         wd = rand(rng, E, d, F, scale=F ** -0.5).to(dt).to(DEV)
         logits = rand(rng, n, E, scale=2.0).to(DEV)
-        tiles = ops.moe_tiles(n * top, E)
+        tiles = ops.moe_tiles(n * top, E, block)
         ids, weights = torch.empty(n * top, dtype=torch.int32, device=DEV), torch.empty(n * top, dtype=torch.float32, device=DEV)
-        rows_list, tile_group = torch.empty(tiles * ops.GROUPED_ROWS, dtype=torch.int32, device=DEV), torch.empty(tiles, dtype=torch.int32, device=DEV)
-        ops.moe_route(logits, top, ids, weights, rows_list, tile_group)
+        rows_list, tile_group = torch.empty(tiles * block, dtype=torch.int32, device=DEV), torch.empty(tiles, dtype=torch.int32, device=DEV)
+        ops.moe_route(logits, top, ids, weights, rows_list, tile_group, block=block)
         inner = torch.full((n * top, F), float("nan"), dtype=dt, device=DEV)
-        ops.moe_product(inner, h, wg, wu, rows_list, tile_group, a_div=top)
+        ops.moe_product(inner, h, wg, wu, rows_list, tile_group, a_div=top, block=block)
         out = torch.full((n * top, d), float("nan"), dtype=torch.float32, device=DEV)
-        ops.moe_product(out, inner, wd, None, rows_list, tile_group, row_scale=weights)
+        ops.moe_product(out, inner, wd, None, rows_list, tile_group, row_scale=weights, block=block)
         hi, e_of, w_of = f64(h), ids.cpu().numpy(), f64(weights)
         want_inner, want = np.zeros((n * top, F)), np.zeros((n * top, d))
         for entry in range(n * top):
