@@ -127,7 +127,7 @@ grouped_mfma_kernel(GroupedParams p) {
         for (int u = 0; u < NW; ++u) w_src[u][i] = w[u] + static_cast<int64_t>(w_ok[i] ? n : 0) * K;
     }
     const gp_u32x4 zero = {0, 0, 0, 0};
-    constexpr int kStages = 4;  // tiles of K whose pieces are in flight: a tile's trip from memory is most of its time otherwise
+    constexpr int kStages = NW == 2 ? 1 : 2;  // tiles of K whose pieces are in flight: a tile's trip from memory is most of its time otherwise
     gp_u32x4 ra[kStages][2], rw[kStages][NW][2];
     auto fetch = [&](int s, int k0) {
         const int k = min(k0 + kc, K - 8);
