@@ -348,10 +348,11 @@ def sequences_run(engine, cfg, counts, prompt_len, n_new, seed=13):
 # -- Bokulix beside GPT-2 at equal sizes ------------------------------------------------------------------
 # Layers that resemble real ones: GPT-2 small's, medium's and XL's widths, head counts and feed-forward widths; the
 # Bokulix of each has the same width, layers, heads (of 64, values of 64), vocabulary and positions, a cached row
-# of 128 (256 at XL's width), a window that covers the context (so that attention walks as many keys), four taps,
-# and experts whose chosen ones together are as wide as GPT-2's feed-forward (top x ff = n_inner).
+# of 128, a window that covers the context (so that attention walks as many keys), four taps, and experts whose
+# chosen ones together are as wide as GPT-2's feed-forward (top x ff = n_inner). (A cached row wider than 128 is
+# taken by the plain attention kernel in prompts: the matrix-core prefill kernel holds heads up to 128.)
 BOKULIX_SHAPES = {"small": {"rank": 128, "experts": 8, "top": 2}, "medium": {"rank": 128, "experts": 16, "top": 2},
-                  "xl": {"rank": 256, "experts": 16, "top": 4}}
+                  "xl": {"rank": 128, "experts": 16, "top": 4}}
 
 
 def bokulix_config(gpt2_cfg, shape):

@@ -14,7 +14,17 @@ namespace liyab {
 
 constexpr int kMaxTaps = 16;
 
-template <typename T>
+typedef __attribute__((ext_vector_type(4))) float conv_f32x4;
+__device__ __forceinline__ void conv_store4(float* dst, const conv_f32x4& v) { *reinterpret_cast<conv_f32x4*>(dst) = v; }
+__device__ __forceinline__ void conv_store4(bf16_t* dst, const conv_f32x4& v) {
+    uint2 packed;
+    packed.x = static_cast<uint32_t>(float_to_bf16(v[0])) | (static_cast<uint32_t>(float_to_bf16(v[1])) << 16);
+    packed.y = static_cast<uint32_t>(float_to_bf16(v[2])) | (static_cast<uint32_t>(float_to_bf16(v[3])) << 16);
+    *reinterpret_cast<uint2*>(dst) = packed;
+}
+
+// VEC: four channels a thread; MAXT: the most taps this instance takes (its earlier inputs are loaded together)
+template <typename T, bool VEC, int MAXT>
 __global__ void __launch_bounds__(256)
 causal_conv_kernel(T* __restrict__ out, T* __restrict__ cast_out, const float* __restrict__ x, const float* __restrict__ w, int taps,
                    const float* __restrict__ state, int n_slots, const int* __restrict__ tok_seq, const int* __restrict__ positions,
@@ -38,6 +48,37 @@ causal_conv_kernel(T* __restrict__ out, T* __restrict__ cast_out, const float* _
         }
     }
     const float* xr = x + static_cast<int64_t>(t) * d;
+    if constexpr (VEC) {
+        // Four channels a thread, 16 bytes a load (d a multiple of 4). Every earlier input is asked for before
+        // any is used, in straight-line code (a load under a branch is waited for where the branch ends, three
+        // trips to memory one after the other): one that does not exist reads this token's own row and counts
+        // as nothing.
+        typedef __attribute__((ext_vector_type(4))) float f32x4;
+        for (int c = (blockIdx.y * 256 + threadIdx.x) * 4; c < d; c += gridDim.y * 1024) {
+            const f32x4 xt = *reinterpret_cast<const f32x4*>(xr + c);
+            const float* wc = w + static_cast<int64_t>(c) * taps;  // the taps of channels c .. c + 3, one after the other
+            f32x4 xm[MAXT - 1];
+            bool there[MAXT - 1];
+#pragma unroll
+            for (int m = 1; m < MAXT; ++m) {
+                there[m - 1] = m <= ring && src[m] != nullptr;
+                xm[m - 1] = *reinterpret_cast<const f32x4*>((there[m - 1] ? src[m] : xr) + c);
+            }
+            f32x4 acc;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[e] = wc[e * taps + taps - 1] * xt[e];
+#pragma unroll
+            for (int m = 1; m < MAXT; ++m)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[e] += there[m - 1] ? wc[e * taps + max(taps - 1 - m, 0)] * xm[m - 1][e] : 0.0f;
+            f32x4 sum;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) sum[e] = xt[e] + acc[e];
+            conv_store4(out + static_cast<int64_t>(t) * d + c, sum);
+            if (cast_out != nullptr) conv_store4(cast_out + static_cast<int64_t>(t) * d + c, xt);
+        }
+        return;
+    }
     for (int c = blockIdx.y * 256 + threadIdx.x; c < d; c += gridDim.y * 256) {
         const float* wc = w + static_cast<int64_t>(c) * taps;
         const float xt = xr[c];
@@ -76,13 +117,22 @@ extern "C" int liyab_causal_conv(void* out, void* cast_out, int dtype, const flo
     LIYAB_REQUIRE(taps == 1 || (state != nullptr && n_slots > 0), "causal_conv: %d taps need the requests' history", taps);
     LIYAB_REQUIRE(dtype == kF32 || dtype == kBF16, "causal_conv: unknown dtype %d", dtype);
     if (n == 0) return 0;
-    const dim3 grid(n, std::min((d + 255) / 256, 64));
-    if (dtype == kF32)
-        causal_conv_kernel<float><<<grid, 256, 0, stream>>>(static_cast<float*>(out), static_cast<float*>(cast_out), x, w, taps, state, n_slots,
-                                                            tok_seq, positions, seq_starts, state_slots, d);
-    else
-        causal_conv_kernel<bf16_t><<<grid, 256, 0, stream>>>(static_cast<bf16_t*>(out), static_cast<bf16_t*>(cast_out), x, w, taps, state,
-                                                             n_slots, tok_seq, positions, seq_starts, state_slots, d);
+    const bool vec = d % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0 &&
+                     (cast_out == nullptr || (reinterpret_cast<uintptr_t>(cast_out) & 15) == 0) && (state == nullptr || (reinterpret_cast<uintptr_t>(state) & 15) == 0);
+    const dim3 grid(n, vec ? std::min((d + 1023) / 1024, 16) : std::min((d + 255) / 256, 64));
+#define LIYAB_CONV(T, V, MAXT)                                                                                                                  \
+    causal_conv_kernel<T, V, MAXT><<<grid, 256, 0, stream>>>(static_cast<T*>(out), static_cast<T*>(cast_out), x, w, taps, state, n_slots, tok_seq, \
+                                                             positions, seq_starts, state_slots, d)
+    if (dtype == kF32) {
+        if (!vec) LIYAB_CONV(float, false, kMaxTaps);
+        else if (taps <= 4) LIYAB_CONV(float, true, 4);
+        else LIYAB_CONV(float, true, kMaxTaps);
+    } else {
+        if (!vec) LIYAB_CONV(bf16_t, false, kMaxTaps);
+        else if (taps <= 4) LIYAB_CONV(bf16_t, true, 4);
+        else LIYAB_CONV(bf16_t, true, kMaxTaps);
+    }
+#undef LIYAB_CONV
     return check_launch("causal_conv");
 }
 
