@@ -17,7 +17,7 @@
 
 namespace liyab {
 
-constexpr int kMaxTop = 32;
+constexpr int kMaxTop = 64;
 
 // One token's choice: the `top` largest of its E logits (the lower number among equals) and the softmax over them.
 __device__ __forceinline__ void route_token(const float* __restrict__ z, int E, int top, int* __restrict__ ids, float* __restrict__ weights) {

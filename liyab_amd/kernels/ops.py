@@ -1163,7 +1163,7 @@ def heads_product(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, gate: Opt
               dtype_code(gate.dtype) if gate is not None else F32, gs, n, N, K, _stream())
 
 
-MOE_MAX_TOP = 32
+MOE_MAX_TOP = 64
 
 
 def moe_tiles(n_entries: int, n_experts: int, block: int = GROUPED_ROWS) -> int:

@@ -20,12 +20,34 @@ from conftest import ROOT, TOL
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 DTYPES = ["float32", "bfloat16"]
-# Relative to the largest |logit| of the compared row, fixed. float32: the families below show 2.5e-6 to
-# 3.8e-6. bfloat16 against the twin in float64 with the same rounded matrices: 4.5e-2 to 5.6e-2, alike
-# whole, in portions, decoded and mixed (a norm stands on every sublayer's result and brings each
-# rounding of a sublayer back to the stream's own size, layer after layer, and these random models'
-# logits lie close together); the tolerance is one and a half times the largest.
-TOL_B = {"float32": TOL["float32"], "bfloat16": 8e-2}
+# float32: the largest difference of a row relative to its largest |logit|, as for the other models; the
+# families below show 2.5e-6 to 7.4e-6 (the largest among the drawn geometries).
+# bfloat16, against the twin in float64 with the same rounded matrices: the root mean square of a row's
+# difference over that of the row's logits, both with their means taken off (what a softmax sees of them).
+# A norm stands on every sublayer's result and brings each rounding of a sublayer back to the stream's own
+# size, layer after layer, and these random models' logits lie close together: single entries of a row are
+# off by up to a tenth of the largest logit (0.045 to 0.11 over the families), which says little; the rows'
+# root mean squares say more: 0.036 to 0.057 for the three geometries below, alike whole, in portions, decoded
+# and mixed, and up to 0.148 among the drawn ones (rows of 8, an epsilon of 1e-3); a fault in a mechanism
+# makes it about 1. Fixed at 0.2.
+TOL_B = {"float32": TOL["float32"], "bfloat16": 2e-1}
+
+
+def check_logits(got, reqs, ref, dtype, what, family=None):
+    """float32: every wanted row within TOL_B of the twin's by its largest entry (trace_tools). bfloat16: by the
+    rows' root mean squares (see above); names the first row that is not."""
+    if dtype == "float32":
+        return tt.check_against_plain(got, reqs, ref, TOL_B[dtype], what, family=family)
+    key = ((family or what.split(" ")[0]) + " (rms)", TOL_B[dtype])
+    for rid, toks in reqs.items():
+        assert rid in got, f"{what}: no logits for request {rid}"
+        for p in sorted(got[rid]):
+            row, want = np.asarray(got[rid][p], dtype=np.float64), ref[rid][p]
+            assert np.isfinite(row).all(), f"{what}: request {rid} position {p}: non-finite logits"
+            diff = row - want
+            e = float(np.sqrt(np.mean((diff - diff.mean()) ** 2)) / np.sqrt(np.mean((want - want.mean()) ** 2)))
+            tt.WORST[key] = max(tt.WORST.get(key, 0.0), e)
+            assert e <= TOL_B[dtype], f"{what}: request {rid} (length {len(toks)}) first differs at position {p}: {e:.3e} > {TOL_B[dtype]:.1e}"
 
 
 def mixer(heads, dim, vdim, rank, window, scale=None):
@@ -431,7 +453,7 @@ def test_each_request_alone_and_whole_and_every_layer(name, dtype, models, refer
     steps = tt.schedule_whole(reqs)
     core = make_core(models[(name, dtype)][0], dtype, tt.max_live_tokens(steps))
     got = tt.run_schedule(core, steps)
-    tt.check_against_plain(got, reqs, reference[(name, dtype)], TOL_B[dtype], f"bokulix-whole {name} {dtype}")
+    check_logits(got, reqs, reference[(name, dtype)], dtype, f"bokulix-whole {name} {dtype}")
     core.manager.check()
     assert core.manager.pages_in_use() == 0
     if dtype == "float32":
@@ -462,7 +484,7 @@ def test_a_prompt_then_its_last_tokens_one_by_one(name, dtype, models, reference
     steps = tt.schedule_bulk_tail(reqs, tail=45)  # past the shorter windows
     core = make_core(models[(name, dtype)][0], dtype, tt.max_live_tokens(steps))
     got = tt.run_schedule(core, steps)
-    tt.check_against_plain(got, reqs, reference[(name, dtype)], TOL_B[dtype], f"bokulix-decode {name} {dtype}")
+    check_logits(got, reqs, reference[(name, dtype)], dtype, f"bokulix-decode {name} {dtype}")
     assert core.manager.pages_in_use() == 0
 
 
@@ -476,7 +498,7 @@ def test_portions_of_changing_size(name, dtype, sizes, models, reference):
     steps = tt.schedule_portions(reqs, sizes)
     core = make_core(models[(name, dtype)][0], dtype, tt.max_live_tokens(steps), page_size=8 if sizes[0] == 1 else 16)
     got = tt.run_schedule(core, steps)
-    tt.check_against_plain(got, reqs, reference[(name, dtype)], TOL_B[dtype], f"bokulix-portions {name} {dtype}")
+    check_logits(got, reqs, reference[(name, dtype)], dtype, f"bokulix-portions {name} {dtype}")
     assert core.manager.pages_in_use() == 0
 
 
@@ -492,7 +514,7 @@ def test_mixed_batches_with_pages_and_slots_used_again(name, dtype, seed, max_li
     steps = tt.schedule_mixed(reqs, seed=seed, max_live=max_live)
     core = make_core(models[(name, dtype)][0], dtype, None, page_size=page_size, max_requests=max_live, num_pages=tt.max_live_pages(steps, page_size))
     got = tt.run_schedule(core, steps)
-    tt.check_against_plain(got, reqs, ref, TOL_B[dtype], f"bokulix-mixed {name} {dtype}")
+    check_logits(got, reqs, ref, dtype, f"bokulix-mixed {name} {dtype}")
     core.manager.check()
     assert core.manager.pages_in_use() == 0
     assert core.step_fn.graph_replays > 0  # the decode-only steps of the tail were replayed from graphs
@@ -507,7 +529,7 @@ def test_long_decoding_from_the_first_token(dtype, models, reference):
     steps = tt.schedule_bulk_tail(reqs, tail=len(toks))
     core = make_core(models[(name, dtype)][0], dtype, tt.max_live_tokens(steps))
     got = tt.run_schedule(core, steps)
-    tt.check_against_plain(got, reqs, reference[(name, dtype)], TOL_B[dtype], f"bokulix-long {dtype}")
+    check_logits(got, reqs, reference[(name, dtype)], dtype, f"bokulix-long {dtype}")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -516,7 +538,69 @@ def test_the_trace_program(dtype, models, reference, tmp_path):
     reqs = make_requests(name)
     steps = tt.schedule_mixed(reqs, seed=5, max_live=4)
     got = tt.run_trace_program(models[(name, dtype)][0], dtype, steps, str(tmp_path), tt.max_live_tokens(steps), CONFIGS[name][0]["vocab"])
-    tt.check_against_plain(got, reqs, reference[(name, dtype)], TOL_B[dtype], f"bokulix-trace {dtype}")
+    check_logits(got, reqs, reference[(name, dtype)], dtype, f"bokulix-trace {dtype}")
+
+
+def draw_config(seed):
+    """A geometry drawn from the seed: every size, window, count and the layers' order."""
+    rng = np.random.default_rng(seed)
+    pick = lambda *options: options[int(rng.integers(len(options)))]  # noqa: E731
+    width = pick(40, 48, 64, 96, 104, 160)
+    layers = []
+    for i in range(int(rng.integers(1, 5))):
+        m = mixer(pick(1, 2, 3, 5, 8), pick(4, 8, 16, 24, 32), pick(8, 12, 16, 40), pick(8, 16, 20, 24, 40, 64, 72, 136),
+                  pick(0, 1, 2, 5, 16, 17, 31, 64, 200))
+        m["scale"] *= pick(0.5, 1.0, 2.0)
+        experts = pick(1, 2, 3, 4, 7, 16, 33)
+        mlp = None if rng.random() < 0.2 else moe(experts, int(rng.integers(1, min(experts, 6) + 1)), pick(8, 20, 24, 40, 56))
+        layers.append(layer(m, mlp))
+    for i in range(int(rng.integers(0, 3))):  # some layers run with an earlier one's tensors, under windows of their own
+        j = int(rng.integers(len(layers)))
+        src = layers[layers[j].get("weights_of", j)]
+        entry = json.loads(json.dumps(src))
+        entry["weights_of"] = layers[j].get("weights_of", j)
+        if rng.random() < 0.5:
+            entry["mixer"]["mask"] = {"size": pick(3, 9, 40)}
+        layers.insert(int(rng.integers(entry["weights_of"] + 1, len(layers) + 1)), entry)
+        for later in layers:  # the layers behind the inserted one have moved up by one
+            if later is not entry and later.get("weights_of") is not None and later["weights_of"] >= layers.index(entry):
+                later["weights_of"] += 1
+    return config(pick(97, 256, 500), width, 320, pick(1e-5, 1e-6, 1e-3), int(rng.integers(1, 7)), layers), pick(8, 16, 24)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_drawn_geometries_whole_and_mixed(seed, tmp_path):
+    """Twelve geometries nobody chose: whole and in mixed batches in a pool just large enough, in 32-bit
+    against the twin; in bfloat16 with every expert chosen (see `every_expert`)."""
+    from liyab_amd.weights import write_random_model
+
+    cfg, page_size = draw_config(seed)
+    for dtype in DTYPES:
+        raw_cfg = every_expert(cfg) if dtype == "bfloat16" else cfg
+        if dtype == "bfloat16":
+            # (scores scaled up make the bfloat16 roundings of queries and cached rows a larger share of a softmax
+            # weight: the drawn factor on the scale is for the 32-bit comparison)
+            for entry in raw_cfg["layers"]:
+                entry["mixer"]["scale"] = 1.0 / math.sqrt(entry["mixer"]["dim"])
+        d = str(tmp_path / dtype)
+        write_random_model(d, json.loads(json.dumps(raw_cfg)), 100 + seed)
+        raw, tensors = plain.read_model(d)
+        t = twin_tensors(tensors, dtype)
+        reqs = {f"g{i}": tt.random_tokens(seed * 10 + i, n, raw["vocab"]) for i, n in enumerate([1, 19, 77, 150, 260])}
+        ref = {rid: plain.forward(raw, t, toks) for rid, toks in reqs.items()}
+        steps = tt.schedule_whole(reqs)
+        core = make_core(d, dtype, tt.max_live_tokens(steps), page_size=page_size)
+        check_logits(tt.run_schedule(core, steps), reqs, ref, dtype, f"bokulix-drawn seed {seed} whole {dtype}", family="bokulix-drawn")
+        steps = tt.schedule_mixed(reqs, seed=seed, max_live=3)
+        core = make_core(d, dtype, None, page_size=page_size, max_requests=3, num_pages=tt.max_live_pages(steps, page_size))
+        check_logits(tt.run_schedule(core, steps), reqs, ref, dtype, f"bokulix-drawn seed {seed} mixed {dtype}", family="bokulix-drawn")
+        core.manager.check()
+        assert core.manager.pages_in_use() == 0
+
+
+# a chosen token's logit in the twin's row lies this close to the row's largest, relative to the largest |logit|
+# (bfloat16: single entries of a row are off by up to 0.11 of it, see TOL_B)
+NEAR_ARGMAX = {"float32": 1e-5, "bfloat16": 1.5e-1}
 
 
 def _near_argmax(row, token, tol):
@@ -542,7 +626,7 @@ def test_greedy_generation_through_the_entry_point(name, dtype, models):
         ref = plain.forward(raw, t, prompt + res.tokens[:-1])
         for i, tok in enumerate(res.tokens):
             row = ref[len(prompt) - 1 + i]
-            assert _near_argmax(row, tok, TOL_B[dtype]), f"token {i} of prompt length {len(prompt)}: {tok} vs {int(np.argmax(row))}"
+            assert _near_argmax(row, tok, NEAR_ARGMAX[dtype]), f"token {i} of prompt length {len(prompt)}: {tok} vs {int(np.argmax(row))}"
         if dtype == "float32":
             assert res.tokens == plain.generate_greedy(raw, t, prompt, n_new)
     assert engine.core.manager.pages_in_use() == 0
