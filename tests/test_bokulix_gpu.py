@@ -598,6 +598,49 @@ def test_drawn_geometries_whole_and_mixed(seed, tmp_path):
         assert core.manager.pages_in_use() == 0
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_sizes_that_are_no_multiple_of_four(dtype, tmp_path):
+    """Width 50, heads of 6 with values of 10, cached rows of 12, experts of 14, a vocabulary of 101: nothing a
+    16-byte load or a matrix instruction takes whole."""
+    from liyab_amd.weights import write_random_model
+
+    cfg = config(101, 50, 200, 1e-5, 3, [layer(mixer(3, 6, 10, 12, 21), moe(5, 2, 14)), layer(mixer(2, 5, 7, 9, 0), moe(3, 3, 6))])
+    cfg = every_expert(cfg) if dtype == "bfloat16" else cfg
+    d = str(tmp_path)
+    write_random_model(d, cfg, 21)
+    raw, tensors = plain.read_model(d)
+    t = twin_tensors(tensors, dtype)
+    reqs = {f"n{i}": tt.random_tokens(300 + i, n, 101) for i, n in enumerate([2, 45, 130])}
+    ref = {rid: plain.forward(raw, t, toks) for rid, toks in reqs.items()}
+    for steps in (tt.schedule_whole(reqs), tt.schedule_mixed(reqs, seed=3, max_live=3)):
+        core = make_core(d, dtype, None, page_size=16, max_requests=3, num_pages=tt.max_live_pages(steps, 16))
+        check_logits(tt.run_schedule(core, steps), reqs, ref, dtype, f"bokulix-narrow {dtype}")
+        assert core.manager.pages_in_use() == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_real_widths_in_long_steps(dtype, tmp_path):
+    """Heads of 64 over cached rows of 128, a window of 300 that prompts of 700 pass twice over, experts of 256: two
+    prompts in one step of 1,400 rows (full tiles of the matrix-core kernels, routing of more than 1,024 tokens), then
+    their last tokens one by one, both requests together."""
+    from liyab_amd.weights import write_random_model
+
+    cfg = config(1000, 256, 1024, 1e-5, 4, [layer(mixer(4, 64, 64, 128, 300), moe(8, 2, 256)), layer(mixer(4, 64, 64, 128, 0), moe(8, 2, 256), weights_of=0)])
+    cfg = every_expert(cfg) if dtype == "bfloat16" else cfg
+    d = str(tmp_path)
+    write_random_model(d, cfg, 22)
+    raw, tensors = plain.read_model(d)
+    t = twin_tensors(tensors, dtype)
+    reqs = {f"w{i}": tt.random_tokens(400 + i, 712, 1000) for i in range(2)}
+    ref = {rid: plain.forward(raw, t, toks) for rid, toks in reqs.items()}
+    want = [0, 1, 299, 300, 301, 511, 512, 699]
+    steps = [{"entries": [(rid, toks[:700], want) for rid, toks in reqs.items()], "end": []}]
+    steps += [{"entries": [(rid, toks[i:i + 1], [0]) for rid, toks in reqs.items()], "end": list(reqs) if i == 711 else []} for i in range(700, 712)]
+    core = make_core(d, dtype, 2 * 768, page_size=16, max_requests=2)
+    check_logits(tt.run_schedule(core, steps), reqs, ref, dtype, f"bokulix-wide {dtype}")
+    assert core.manager.pages_in_use() == 0
+
+
 # a chosen token's logit in the twin's row lies this close to the row's largest, relative to the largest |logit|
 # (bfloat16: single entries of a row are off by up to 0.11 of it, see TOL_B)
 NEAR_ARGMAX = {"float32": 1e-5, "bfloat16": 1.5e-1}
