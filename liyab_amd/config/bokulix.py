@@ -8,8 +8,8 @@ norms; a final norm and an untied head. config.json:
     architecture   "Bokulix"
     vocab, width, max_positions
     norm.eps       the epsilon of every norm of a layer, of the final norm and of the cached row's
-    canon.taps     the taps of the input convolution
-    layers[i]      type ("latent_attention"), mixer {heads, dim, vdim, kv_rank, scale, mask.size},
+    canon.taps     the taps of the input convolution (no `canon`: none)
+    layers[i]      type ("latent_attention"), mixer {heads, dim, vdim, kv_rank, scale, mask.size (no `mask`: every earlier position)},
                    mlp (null, or {kind "moe", expert.ff, router.experts, router.top}),
                    weights_of (optional): the layer whose tensors this one runs with, its cache and
                    state being its own
@@ -95,7 +95,7 @@ class BokulixConfig:
         vocab, width = _int(raw, "vocab", "vocab"), _int(raw, "width", "width")
         max_positions = _int(raw, "max_positions", "max_positions")
         eps = _number(raw.get("norm"), "eps", "norm.eps")
-        taps = _int(raw.get("canon"), "taps", "canon.taps")
+        taps = _int(raw.get("canon"), "taps", "canon.taps") if raw.get("canon") is not None else 0  # (no entry: no input convolution)
         listed = raw.get("layers")
         if not isinstance(listed, list) or not listed:
             raise InvalidModel("missing or invalid layers")
@@ -109,7 +109,7 @@ class BokulixConfig:
             m = entry.get("mixer")
             where = f"layers[{i}].mixer"
             mask = m.get("mask") if isinstance(m, dict) else None
-            window = _int(mask, "size", where + ".mask.size") if mask is not None else 0
+            window = _int(mask, "size", where + ".mask.size") if mask is not None and (not isinstance(mask, dict) or mask.get("size") is not None) else 0
             mlp = entry.get("mlp")
             routed = None
             if mlp is not None:
@@ -154,8 +154,11 @@ class BokulixConfig:
             if layer.weights_of is not None:
                 entry["weights_of"] = layer.weights_of
             layers.append(entry)
-        return {"architecture": self.architecture, "vocab": self.vocab, "width": self.width, "max_positions": self.max_positions,
-                "norm": {"eps": self.eps}, "canon": {"taps": self.taps}, "layers": layers}
+        out = {"architecture": self.architecture, "vocab": self.vocab, "width": self.width, "max_positions": self.max_positions,
+               "norm": {"eps": self.eps}, "layers": layers}
+        if self.taps:
+            out["canon"] = {"taps": self.taps}
+        return out
 
     def plan(self) -> ModelPlan:
         d, V = self.width, self.vocab
@@ -200,7 +203,7 @@ class BokulixConfig:
                 mixer=mixer, ffn=ffn, norm_mixer=norm(p + ".norm1"), norm_ffn=norm(p + ".norm2") if ffn is not None else None,
                 arrangement="post_norm_gated",
                 input_conv=CausalConvSpec(kind="causal_conv", width=d, taps=self.taps,
-                                          tensors={"weight": TensorSource(p + ".canon1", init=Init(0.3))}),
+                                          tensors={"weight": TensorSource(p + ".canon1", init=Init(0.3))}) if self.taps else None,
                 gate_mixer=gate(p + ".rg1"), gate_ffn=gate(p + ".rg2") if ffn is not None else None))
         return ModelPlan(
             architecture=self.architecture, width=d, vocab_size=V, max_positions=self.max_positions,

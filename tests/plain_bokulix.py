@@ -101,7 +101,8 @@ def layer(x, t, config, i):
     entry = config["layers"][i]
     p = f"l{entry.get('weights_of', i) if entry.get('weights_of') is not None else i}."
     eps = config["norm"]["eps"]
-    y = latent_attention(input_convolution(x, t[p + "canon1"]), t, p + "mix.", entry["mixer"], eps)
+    u = input_convolution(x, t[p + "canon1"]) if config.get("canon") is not None else x
+    y = latent_attention(u, t, p + "mix.", entry["mixer"], eps)
     x = x + rms(y * sigmoid(x @ t[p + "rg1"].T + t[p + "rg1.b"]), t[p + "norm1"], eps)
     if entry.get("mlp") is not None:
         y = routed_experts(x, t, p + "mlp.", entry["mlp"])

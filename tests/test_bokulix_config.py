@@ -32,6 +32,17 @@ def test_config_round_trip_and_plan():
     assert plan.final_norm.kind == "rmsnorm" and plan.head.tensors["weight"].name == "head"
 
 
+def test_what_may_be_left_out():
+    raw = raw_config()
+    del raw["canon"]
+    raw["layers"][0]["mixer"]["mask"] = None
+    raw["layers"][1]["mixer"]["mask"] = {"size": None}
+    cfg = config_from_dict(raw)
+    assert cfg.taps == 0 and [l.window for l in cfg.layers[:2]] == [0, 0]
+    assert all(l.input_conv is None for l in cfg.plan().layers)
+    assert config_from_dict(cfg.to_json()) == cfg
+
+
 def test_random_weights_name_every_tensor_once():
     from liyab_amd.weights.random_init import random_tensors
 

@@ -598,13 +598,16 @@ def test_drawn_geometries_whole_and_mixed(seed, tmp_path):
         assert core.manager.pages_in_use() == 0
 
 
+@pytest.mark.parametrize("convolved", [True, False])
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_sizes_that_are_no_multiple_of_four(dtype, tmp_path):
+def test_sizes_that_are_no_multiple_of_four(dtype, convolved, tmp_path):
     """Width 50, heads of 6 with values of 10, cached rows of 12, experts of 14, a vocabulary of 101: nothing a
-    16-byte load or a matrix instruction takes whole."""
+    16-byte load or a matrix instruction takes whole. Also without the input convolution (no `canon` entry)."""
     from liyab_amd.weights import write_random_model
 
     cfg = config(101, 50, 200, 1e-5, 3, [layer(mixer(3, 6, 10, 12, 21), moe(5, 2, 14)), layer(mixer(2, 5, 7, 9, 0), moe(3, 3, 6))])
+    if not convolved:
+        del cfg["canon"]
     cfg = every_expert(cfg) if dtype == "bfloat16" else cfg
     d = str(tmp_path)
     write_random_model(d, cfg, 21)
