@@ -47,7 +47,7 @@ class TensorSource:
 
 @dataclass(frozen=True)
 class NormSpec:
-    kind: str  # "layernorm" | "rmsnorm" (weight only)
+    kind: str  # "layernorm" | "rmsnorm" (weight only) | "dyt" (tanh(alpha x) * weight + bias: tensors weight, bias, alpha)
     width: int
     eps: float
     tensors: dict = field(default_factory=dict)  # "weight", "bias"
@@ -154,10 +154,114 @@ class GateSpec:
 
 
 @dataclass(frozen=True)
+class RotarySpec:
+    """Pairs (2i, 2i + 1) of the first `dims` entries of a head turned by position * f_i, f_i = base^(-2i / dims);
+    `scaling` (factor, low, high, original) stretches the long wavelengths: f stays where the wavelength is under
+    original / high, becomes f / factor where it is over original / low, and is blended in between."""
+
+    dims: int
+    base: float
+    scaling: Optional[tuple] = None  # (factor, low, high, original)
+
+
+@dataclass(frozen=True)
+class ScoredAttentionSpec:
+    """Attention over paged keys and values whose queries, keys and scores are worked on: keys `head_dim` wide, values
+    `value_dim`; each of these optional: a root-mean-square norm of every query and key head (`qk_norm`, weights shared by
+    the heads), a rotary encoding (`rotary`), a factor on the query that grows with the position's logarithm (`q_temp` =
+    (coef, every): 1 + coef * ln(floor((p + 1) / every) + 1)), a soft cap on the scores (`softcap`: cap * tanh(score / cap)),
+    a learned bias by distance (`distance_bias` = the distance from which the table's last row holds; the table's rows:
+    the distance itself below half of them, then logarithmic steps), values that are the keys as projected
+    (`values_are_keys`), a sigmoid gate on the heads' results from a projection of the mixer's input (`gated`)."""
+
+    kind: str  # "scored_attention"
+    width: int
+    n_head: int
+    n_kv_head: int
+    head_dim: int
+    value_dim: int
+    scale: float
+    eps: float
+    window: int = 0
+    softcap: float = 0.0
+    qk_norm: bool = False
+    rotary: Optional[RotarySpec] = None
+    q_temp: Optional[tuple] = None  # (coef, every)
+    distance_bias: int = 0  # 0: none
+    bias_rows: int = 0
+    values_are_keys: bool = False
+    gated: bool = False
+    tensors: dict = field(default_factory=dict)  # q, k, v, gate, out, q_norm, k_norm, rel
+
+
+@dataclass(frozen=True)
+class WKVSpec:
+    """A mixer that carries a matrix of state a head: five learned mixes of a token's input with the one before it feed
+    receptance, key, value, gate and a low-rank decay (`decay_rank` wide); o = (S + diag(u) k v^T)^T r, S <- diag(w) S + k v^T;
+    each head's result brought to unit root mean square, times a weight and silu(gate), then the output projection."""
+
+    kind: str  # "wkv"
+    width: int
+    n_head: int
+    head_dim: int
+    decay_rank: int
+    eps: float
+    tensors: dict = field(default_factory=dict)  # mu_r, mu_k, mu_v, mu_g, mu_w, r, k, v, g, w1, w2, w0, u, norm, out
+
+
+@dataclass(frozen=True)
+class StateSpaceSpec:
+    """A selective state-space mixer: one projection gives [z | x | B | C | dt]; x, B and C pass a short causal convolution
+    (`taps`) with a bias and silu; per head S <- exp(-exp(A_log) dt) S + dt B x^T with dt = softplus(dt + dt_bias), y = S^T C +
+    D x; y * silu(z) is brought to unit root mean square in `norm_groups` equal parts, times a weight, then the output
+    projection. Heads share B and C in `n_groups` groups."""
+
+    kind: str  # "state_space"
+    width: int
+    n_head: int
+    head_dim: int
+    n_state: int
+    n_groups: int
+    taps: int
+    norm_groups: int
+    eps: float
+    tensors: dict = field(default_factory=dict)  # in, conv, conv_bias, dt_bias, A_log, D, norm, out
+
+
+@dataclass(frozen=True)
+class SideBySideSpec:
+    """Two mixers that read the same input; the result is `weight` times the sum of their results, each brought to unit
+    root mean square over the model's width first and multiplied by a weight of its own."""
+
+    kind: str  # "side_by_side"
+    width: int
+    left: Any
+    right: Any
+    eps: float
+    weight: float = 0.5
+    tensors: dict = field(default_factory=dict)  # left_out, right_out
+
+
+@dataclass(frozen=True)
+class ClampedGLUSpec:
+    """A gated feed-forward whose halves are clamped before they meet: g = min(Wg h, limit), u = clamp(Wu h, -limit, limit),
+    down(g * sigmoid(slope * g) * (u + shift))."""
+
+    kind: str  # "clamped_glu"
+    width: int
+    inner: int
+    limit: float
+    slope: float = 1.702
+    shift: float = 1.0
+    tensors: dict = field(default_factory=dict)  # gate, up, down
+
+
+@dataclass(frozen=True)
 class LayerSpec:
     """One block: which parts it has and how they are arranged.
 
     arrangement "pre_norm": x += mixer(norm_mixer(x)); x += ffn(norm_ffn(x)).
+    arrangement "parallel": h = norm_mixer(x); x += mixer(h) + ffn(h): one norm, both sublayers read its output.
     arrangement "post_norm_gated": x += norm_mixer(gate_mixer * mixer(conv(x))); x += norm_ffn(gate_ffn *
     ffn(x)): the sublayers read the stream itself, the norms stand on their results; `input_conv`
     (what the mixer reads is first convolved over time) and the gates are optional.

@@ -9,6 +9,7 @@ itself is always the generic decoder built from the plan.
 
 from __future__ import annotations
 
+import inspect
 import json
 import os
 from typing import Callable, Dict, List
@@ -57,11 +58,15 @@ def architecture_name_of(raw: dict) -> str:
     raise InvalidModel("not a model folder: config.json has neither 'architectures' nor 'architecture' nor 'model_type'")
 
 
-def config_from_dict(raw: dict):
-    """Typed configuration for a parsed config.json."""
+def config_from_dict(raw: dict, shapes=None):
+    """Typed configuration for a parsed config.json. `shapes` (tensor name -> shape, of the weights file beside it) goes
+    to configuration classes that read sizes from tensors' shapes (`from_json(raw, shapes=)`)."""
     if not isinstance(raw, dict):
         raise InvalidModel("config.json must hold a JSON object")
-    return find_architecture(architecture_name_of(raw)).from_json(raw)
+    cls = find_architecture(architecture_name_of(raw))
+    if shapes is not None and "shapes" in inspect.signature(cls.from_json).parameters:
+        return cls.from_json(raw, shapes=shapes)
+    return cls.from_json(raw)
 
 
 def load_config(model_dir: str):
@@ -73,4 +78,10 @@ def load_config(model_dir: str):
             raw = json.load(f)
     except json.JSONDecodeError as e:
         raise InvalidModel(f"config.json is not valid JSON: {e}") from None
-    return config_from_dict(raw)
+    shapes = None
+    weights = os.path.join(model_dir, "model.safetensors")
+    if os.path.isfile(weights):
+        from ..weights.safetensors_io import SafetensorsFile
+
+        shapes = {name: e.shape for name, e in SafetensorsFile(weights).entries.items()}
+    return config_from_dict(raw, shapes)

@@ -1,0 +1,223 @@
+// Attention whose scores are more than scale * q . k, over paged keys and values of widths of their own.
+//
+// liyab_qk_prepare: what happens to a step's projected queries, keys and values between the projection
+// and the cache. The source is the projection's 32-bit output [q heads | ... | k heads | ... | v heads]
+// (values may be the keys' own columns: values that are the keys as projected). Per head, in this
+// order: a root-mean-square norm over the head with a weight shared by all heads (queries and keys,
+// each optional); the turning of pairs (2i, 2i + 1) of the first `rot_dims` entries by position * f_i
+// (queries and keys; f from a table); a factor on the query that grows with the logarithm of the
+// position, 1 + coef * ln(floor((p + 1) / every) + 1). Queries go to a dense buffer in the compute type,
+// keys and values to their token's slot of the pages. Norms, angles and factors are 32-bit.
+//
+// liyab_attention_scored: one workgroup a (token, query head). score = scale * q . k, then, each optional:
+// a soft cap, cap * tanh(score / cap); a learned bias by distance, table[min(i - j, max_dist), head].
+// Causal, with an optional window; ordinary softmax in 32-bit over tiles of 256 keys in position order
+// with a running maximum and sum, so that a row's rounding follows from its position alone. Values are
+// `dv` wide (keys `dk`). The result may be multiplied by the logistic function of a gate's logits before
+// it is rounded to the compute type.
+#include "common.h"
+#include "launchers.h"
+
+namespace liyab {
+
+constexpr int AS_THREADS = 256;
+
+template <typename T>
+__global__ void __launch_bounds__(kWave)
+qk_prepare_kernel(const float* __restrict__ src, int64_t ld, int q_off, int k_off, int v_off, int H, int G, int dk, int dv,
+                  T* __restrict__ q_out, T* __restrict__ kc, T* __restrict__ vc, const int* __restrict__ slots, int page_size,
+                  int num_pages, const float* __restrict__ q_norm, const float* __restrict__ k_norm, float eps,
+                  const float* __restrict__ freqs, int rot_dims, float temp_coef, int temp_every, const int* __restrict__ positions) {
+    const int t = blockIdx.x, hh = blockIdx.y, lane = threadIdx.x;
+    const int p = positions[t];
+    const float* row = src + static_cast<int64_t>(t) * ld;
+    if (hh < H + G) {
+        const bool is_q = hh < H;
+        const int head = is_q ? hh : hh - H;
+        const float* x = row + (is_q ? q_off : k_off) + head * dk;
+        const float* nw = is_q ? q_norm : k_norm;
+        float factor = 1.0f;
+        if (nw != nullptr) {
+            float ss = 0.0f;
+            for (int i = lane; i < dk; i += kWave) ss = fmaf(x[i], x[i], ss);
+            factor = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(dk) + eps);
+        }
+        float temp = 1.0f;
+        if (is_q && temp_every > 0) temp = 1.0f + temp_coef * logf(static_cast<float>((p + 1) / temp_every) + 1.0f);
+        T* dst;
+        if (is_q) {
+            dst = q_out + static_cast<int64_t>(t) * H * dk + head * dk;
+        } else {
+            const int64_t slot = slots[t];
+            if (slot < 0 || slot >= static_cast<int64_t>(num_pages) * page_size) return;
+            dst = kc + (((slot / page_size) * G + head) * page_size + slot % page_size) * dk;
+        }
+        // pairs of entries: a lane takes a pair at a time
+        for (int i2 = lane; 2 * i2 < dk; i2 += kWave) {
+            const int e0 = 2 * i2, e1 = e0 + 1;
+            float a = x[e0] * factor * (nw != nullptr ? nw[e0] : 1.0f);
+            float b = e1 < dk ? x[e1] * factor * (nw != nullptr ? nw[e1] : 1.0f) : 0.0f;
+            if (freqs != nullptr && e1 < rot_dims) {
+                const float angle = static_cast<float>(p) * freqs[i2];
+                const float c = cosf(angle), s = sinf(angle);
+                const float ra = a * c - b * s, rb = b * c + a * s;
+                a = ra;
+                b = rb;
+            }
+            dst[e0] = from_float<T>(a * temp);
+            if (e1 < dk) dst[e1] = from_float<T>(b * temp);
+        }
+    } else {
+        const int head = hh - H - G;
+        const int64_t slot = slots[t];
+        if (slot < 0 || slot >= static_cast<int64_t>(num_pages) * page_size) return;
+        const float* x = row + v_off + head * dv;
+        T* dst = vc + (((slot / page_size) * G + head) * page_size + slot % page_size) * dv;
+        for (int i = lane; i < dv; i += kWave) dst[i] = from_float<T>(x[i]);
+    }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(AS_THREADS)
+attention_scored_kernel(T* __restrict__ out, int64_t out_stride, const T* __restrict__ q, int64_t q_stride, const T* __restrict__ kc,
+                        const T* __restrict__ vc, const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ tok_seq,
+                        const int* __restrict__ tok_pos, float scale, float softcap, int window, const float* __restrict__ bias_table,
+                        int max_dist, const float* __restrict__ gate, int64_t gate_stride, int n_head, int n_kv_head, int dk, int dv,
+                        int page_size, int num_pages) {
+    extern __shared__ float smem[];
+    float* qs = smem;                          // [dk]
+    float* sc = qs + dk;                       // [AS_THREADS]
+    float* red = sc + AS_THREADS;              // [AS_THREADS / kWave]
+    float* accs = red + AS_THREADS / kWave;    // [G][dv]
+
+    const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+    const int wave = tid / kWave, lane = tid % kWave;
+    const int pos = static_cast<int>(min(static_cast<int64_t>(max(tok_pos[t], 0)), static_cast<int64_t>(max_blocks) * page_size - 1));
+    const int* bt = block_tables + static_cast<int64_t>(tok_seq[t]) * max_blocks;
+    const int hkv = h / (n_head / n_kv_head);
+    const int first = window > 0 ? max(0, pos - window + 1) : 0;
+    const T* qrow = q + static_cast<int64_t>(t) * q_stride + static_cast<int64_t>(h) * dk;
+    for (int e = tid; e < dk; e += AS_THREADS) qs[e] = to_float<T>(qrow[e]);
+    __syncthreads();
+
+    const int G = AS_THREADS / dv;  // groups of dv threads sharing the keys of a tile
+    const int g = tid / dv, e = tid % dv;
+    const bool vthread = g < G;
+    const float inv_cap = softcap > 0.0f ? 1.0f / softcap : 0.0f;
+    float m = -INFINITY, l = 0.0f, acc = 0.0f;
+
+    for (int j0 = first; j0 <= pos; j0 += AS_THREADS) {
+        const int j = j0 + tid;
+        float s = -INFINITY;
+        if (j <= pos) {
+            const int64_t page = min(max(bt[j / page_size], 0), num_pages - 1);
+            const T* kr = kc + ((page * n_kv_head + hkv) * page_size + j % page_size) * dk;
+            float dot = 0.0f;
+            for (int i = 0; i < dk; ++i) dot = fmaf(to_float<T>(kr[i]), qs[i], dot);
+            s = dot * scale;
+            if (softcap > 0.0f) s = softcap * tanhf(s * inv_cap);
+            if (bias_table != nullptr) s += bias_table[static_cast<int64_t>(min(pos - j, max_dist)) * n_head + h];
+        }
+        float tm = wave_max(s);
+        if (lane == 0) red[wave] = tm;
+        __syncthreads();
+        tm = red[0];
+#pragma unroll
+        for (int i = 1; i < AS_THREADS / kWave; ++i) tm = fmaxf(tm, red[i]);
+        const float m_new = fmaxf(m, tm);
+        const float p = j <= pos ? expf(s - m_new) : 0.0f;
+        sc[tid] = p;
+        float ps = wave_sum(p);
+        __syncthreads();
+        if (lane == 0) red[wave] = ps;
+        __syncthreads();
+        ps = 0.0f;
+#pragma unroll
+        for (int i = 0; i < AS_THREADS / kWave; ++i) ps += red[i];
+        const float corr = expf(m - m_new);
+        l = l * corr + ps;
+        acc *= corr;
+        m = m_new;
+        if (vthread) {
+            const int len = min(AS_THREADS, pos - j0 + 1);
+            for (int jj = g; jj < len; jj += G) {
+                const int jv = j0 + jj;
+                const int64_t page = min(max(bt[jv / page_size], 0), num_pages - 1);
+                const T* vr = vc + ((page * n_kv_head + hkv) * page_size + jv % page_size) * dv;
+                acc = fmaf(sc[jj], to_float<T>(vr[e]), acc);
+            }
+        }
+        __syncthreads();
+    }
+    if (vthread) accs[g * dv + e] = acc;
+    __syncthreads();
+    if (tid < dv) {
+        float o = 0.0f;
+        for (int i = 0; i < G; ++i) o += accs[i * dv + tid];
+        o /= l;
+        if (gate != nullptr) o *= 1.0f / (1.0f + expf(-gate[static_cast<int64_t>(t) * gate_stride + static_cast<int64_t>(h) * dv + tid]));
+        out[static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * dv + tid] = from_float<T>(o);
+    }
+}
+
+}  // namespace liyab
+
+using namespace liyab;
+
+extern "C" int liyab_qk_prepare(const float* src, int64_t ld, int q_off, int k_off, int v_off, int H, int G, int dk, int dv, void* q_out,
+                                void* kc, void* vc, int dtype, const int* slots, int page_size, int num_pages, const float* q_norm,
+                                const float* k_norm, float eps, const float* freqs, int rot_dims, float temp_coef, int temp_every,
+                                const int* positions, int n, hipStream_t stream) {
+    LIYAB_REQUIRE(src && q_out && kc && vc && slots && positions, "qk_prepare: null pointer");
+    LIYAB_REQUIRE(n >= 0 && H > 0 && G > 0 && dk > 0 && dv > 0 && page_size > 0 && num_pages > 0, "qk_prepare: bad sizes");
+    LIYAB_REQUIRE(H + 2 * G <= 65535, "qk_prepare: too many heads");
+    LIYAB_REQUIRE(q_off >= 0 && k_off >= 0 && v_off >= 0 && q_off + static_cast<int64_t>(H) * dk <= ld && k_off + static_cast<int64_t>(G) * dk <= ld &&
+                      v_off + static_cast<int64_t>(G) * dv <= ld,
+                  "qk_prepare: the heads' columns pass the source's rows");
+    LIYAB_REQUIRE(rot_dims >= 0 && rot_dims <= dk && rot_dims % 2 == 0 && (rot_dims == 0 || freqs != nullptr), "qk_prepare: %d turned entries of heads of %d", rot_dims, dk);
+    LIYAB_REQUIRE(temp_every >= 0, "qk_prepare: bad query factor");
+    if (n == 0) return 0;
+    dim3 grid(n, H + 2 * G);
+    const float* fr = rot_dims > 0 ? freqs : nullptr;
+    if (dtype == kF32)
+        qk_prepare_kernel<float><<<grid, kWave, 0, stream>>>(src, ld, q_off, k_off, v_off, H, G, dk, dv, static_cast<float*>(q_out), static_cast<float*>(kc),
+                                                             static_cast<float*>(vc), slots, page_size, num_pages, q_norm, k_norm, eps, fr, rot_dims,
+                                                             temp_coef, temp_every, positions);
+    else if (dtype == kBF16)
+        qk_prepare_kernel<bf16_t><<<grid, kWave, 0, stream>>>(src, ld, q_off, k_off, v_off, H, G, dk, dv, static_cast<bf16_t*>(q_out),
+                                                              static_cast<bf16_t*>(kc), static_cast<bf16_t*>(vc), slots, page_size, num_pages, q_norm,
+                                                              k_norm, eps, fr, rot_dims, temp_coef, temp_every, positions);
+    else return fail(1, "qk_prepare: unknown dtype %d", dtype);
+    return check_launch("qk_prepare");
+}
+
+extern "C" int liyab_attention_scored(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc, const void* vc, int dtype,
+                                      const int* block_tables, int max_blocks, const int* tok_seq, const int* tok_pos, int n, float scale,
+                                      float softcap, int window, const float* bias_table, int max_dist, const float* gate, int64_t gate_stride,
+                                      int n_head, int n_kv_head, int dk, int dv, int page_size, int num_pages, hipStream_t stream) {
+    LIYAB_REQUIRE(out && q && kc && vc && block_tables && tok_seq && tok_pos, "attention_scored: null pointer");
+    LIYAB_REQUIRE(num_pages > 0 && n >= 0 && n_head > 0 && n_kv_head > 0 && page_size > 0 && max_blocks > 0, "attention_scored: bad sizes");
+    LIYAB_REQUIRE(n_head % n_kv_head == 0, "attention_scored: %d query heads are no multiple of %d key/value heads", n_head, n_kv_head);
+    LIYAB_REQUIRE(dk > 0 && dk <= 512 && dv > 0 && dv <= AS_THREADS, "attention_scored: heads of %d / %d are outside 1..512 / 1..256", dk, dv);
+    LIYAB_REQUIRE(out_stride >= static_cast<int64_t>(n_head) * dv && q_stride >= static_cast<int64_t>(n_head) * dk, "attention_scored: row strides are shorter than the heads");
+    LIYAB_REQUIRE(window >= 0 && softcap >= 0.0f, "attention_scored: negative window or cap");
+    LIYAB_REQUIRE(bias_table == nullptr || max_dist >= 0, "attention_scored: a bias table needs its largest distance");
+    LIYAB_REQUIRE(gate == nullptr || gate_stride >= static_cast<int64_t>(n_head) * dv, "attention_scored: the gate's rows are shorter than the heads");
+    LIYAB_REQUIRE(n_head <= 65535, "attention_scored: too many heads");
+    if (n == 0) return 0;
+    const int G = AS_THREADS / dv;
+    const size_t smem = sizeof(float) * (dk + AS_THREADS + AS_THREADS / kWave + static_cast<size_t>(G) * dv);
+    dim3 grid(n, n_head);
+    if (dtype == kF32)
+        attention_scored_kernel<float><<<grid, AS_THREADS, smem, stream>>>(
+            static_cast<float*>(out), out_stride, static_cast<const float*>(q), q_stride, static_cast<const float*>(kc), static_cast<const float*>(vc),
+            block_tables, max_blocks, tok_seq, tok_pos, scale, softcap, window, bias_table, max_dist, gate, gate_stride, n_head, n_kv_head, dk, dv,
+            page_size, num_pages);
+    else if (dtype == kBF16)
+        attention_scored_kernel<bf16_t><<<grid, AS_THREADS, smem, stream>>>(
+            static_cast<bf16_t*>(out), out_stride, static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(kc), static_cast<const bf16_t*>(vc),
+            block_tables, max_blocks, tok_seq, tok_pos, scale, softcap, window, bias_table, max_dist, gate, gate_stride, n_head, n_kv_head, dk, dv,
+            page_size, num_pages);
+    else return fail(1, "attention_scored: unknown dtype %d", dtype);
+    return check_launch("attention_scored");
+}

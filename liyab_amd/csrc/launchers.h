@@ -79,4 +79,37 @@ int liyab_moe_route_align(const float* logits, int64_t ld, int n, int n_experts,
 int liyab_moe_align(const int* ids, int n_entries, int n_experts, int block, int* rows_list, int* tile_group, int max_tiles,
                     hipStream_t stream);
 
+int liyab_dyt(void* out, int out_dtype, const float* x, const float* w, const float* b, const float* alpha, const int* rows, int n, int d,
+              hipStream_t stream);
+int liyab_glu_clamped(void* out, int out_dtype, const float* gu, int64_t ld, int n, int ff, float limit, float slope, float shift,
+                      hipStream_t stream);
+int liyab_activate(void* out, int out_dtype, int64_t ldo, const float* in, int64_t ldi, int op, int n, int d, hipStream_t stream);
+int liyab_mean_norm_add(float* x, const float* a, const float* b, const float* wa, const float* wb, float eps, float weight, int n, int d,
+                        hipStream_t stream);
+int liyab_scan_takes(int rows, int cols);
+int liyab_wkv_scan(void* out, int out_dtype, const float* r, const float* k, const float* v, const float* wraw, const float* gate, int64_t ld,
+                   const float* w0, const float* u, const float* norm_w, float eps, float* state, int64_t state_stride, int n_slots,
+                   const void* keep_src, int keep_dtype, int64_t keep_ld, int keep_width, int64_t keep_off, const int* seq_starts,
+                   const int* positions, const int* state_slots, int n_seqs, int H, int D, hipStream_t stream);
+int liyab_ssd_scan(float* y, int64_t ldy, const float* xbc, int64_t ldx, const float* dtraw, int64_t ldp, const float* dt_bias,
+                   const float* A_log, const float* Dskip, float* state, int64_t state_stride, int n_slots, const float* keep_src,
+                   int64_t keep_ld, int keep_width, int keep_ring, int64_t keep_off, const int* seq_starts, const int* positions,
+                   const int* state_slots, int n_seqs, int H, int P, int N, int G, hipStream_t stream);
+int liyab_token_shift(void* out, int dtype, const void* h, const float* mu, int n_mix, const float* state, int64_t state_stride, int n_slots,
+                      const int* tok_seq, const int* positions, const int* seq_starts, const int* state_slots, int n, int d,
+                      hipStream_t stream);
+int liyab_conv_act(float* out, int64_t ldo, const float* in, int64_t ldi, const float* w, const float* bias, int taps, const float* state,
+                   int64_t state_stride, int n_slots, const int* tok_seq, const int* positions, const int* seq_starts,
+                   const int* state_slots, int n, int C, hipStream_t stream);
+int liyab_gated_group_norm(void* out, int out_dtype, const float* y, int64_t ldy, const float* z, int64_t ldz, const float* w, float eps,
+                           int n, int inner, int groups, hipStream_t stream);
+int liyab_qk_prepare(const float* src, int64_t ld, int q_off, int k_off, int v_off, int H, int G, int dk, int dv, void* q_out, void* kc,
+                     void* vc, int dtype, const int* slots, int page_size, int num_pages, const float* q_norm, const float* k_norm,
+                     float eps, const float* freqs, int rot_dims, float temp_coef, int temp_every, const int* positions, int n,
+                     hipStream_t stream);
+int liyab_attention_scored(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc, const void* vc, int dtype,
+                           const int* block_tables, int max_blocks, const int* tok_seq, const int* tok_pos, int n, float scale,
+                           float softcap, int window, const float* bias_table, int max_dist, const float* gate, int64_t gate_stride,
+                           int n_head, int n_kv_head, int dk, int dv, int page_size, int num_pages, hipStream_t stream);
+
 }  // extern "C"

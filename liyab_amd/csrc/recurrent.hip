@@ -1,0 +1,414 @@
+// Mixers that carry a matrix of state from token to token instead of keys: the recurrence itself and
+// what stands around it.
+//
+// Both recurrences here keep, a head, a matrix S [rows, cols] of 32-bit floats a request:
+//   decayed outer products with a bonus (a "wkv" head; rows = key channels, cols = value channels):
+//       o_t = (S + diag(u) k_t v_t^T)^T r_t,      S <- diag(w_t) S + k_t v_t^T,   w_t = exp(-exp(wraw_t + w0))
+//   a selective state space (rows = state size, cols = the head's channels), a = exp(-exp(A_log) dt_t):
+//       S <- a S + dt_t B_t x_t^T,                y_t = S^T C_t + D x_t,          dt_t = softplus(dtraw_t + dt_bias)
+// One kernel serves both: a workgroup a (request, head) walks the request's tokens of the step in order.
+// A thread owns one column of a block of rows of S in registers, so nothing of the state moves between
+// threads; a token's vectors are staged through LDS sixteen tokens at a time (one trip to memory a
+// chunk, not a token), the threads leave partial sums of the outputs in LDS, and after the chunk the
+// workgroup adds them up and finishes the rows (a wkv head: unit root mean square over the head, the
+// weight, the gate silu(g); a state-space head: + D x). The state comes from the request's slot (zeros
+// at position 0 whatever the slot still holds) and goes back to it. The workgroup of head 0 also keeps
+// the request's last input rows for the next step (the previous token's input of a token shift, the last
+// taps - 1 inputs of a short convolution), at ring place position % ring: after every read of them, since
+// the kernels that read them ran before this one.
+//
+// liyab_token_shift: m_c[t] = h[t] + (h[t - 1] - h[t]) * mu_c for each of n_mix learned mixes, the previous
+//   row taken from the step's rows, from the request's slot, or zero at position 0.
+// liyab_conv_act: out[t, c] = silu(bias[c] + sum_j w[c, j] * in[t - taps + 1 + j, c]) over a request's
+//   own rows in time (the last column of w is the current row's), earlier rows from the ring.
+// liyab_gated_group_norm: out = unit_rms_g(y * silu(z)) * w, the root mean square taken over each of
+//   `groups` equal parts of a row.
+#include "common.h"
+#include "launchers.h"
+
+namespace liyab {
+
+constexpr int SCAN_THREADS = 256;
+constexpr int SCAN_CHUNK = 16;  // tokens staged through LDS together
+
+__device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z)); }
+__device__ __forceinline__ float softplus_f(float z) { return z > 20.0f ? z : log1pf(expf(z)); }
+
+struct ScanArgs {
+    // common
+    float* state;           // [n_slots, state_stride]; the heads' matrices first, [H, rows, cols]
+    int64_t state_stride;
+    int n_slots;
+    const int* seq_starts;  // [n_seqs + 1]
+    const int* positions;   // [n]
+    const int* state_slots; // [n_seqs]
+    int H, rows, cols;
+    int col_lanes;          // a power of two >= cols (threads side by side a block of rows)
+    int rows_per;           // rows a thread holds
+    // the rows kept for the next step
+    const void* keep_src;
+    int keep_bf16;
+    int64_t keep_ld;
+    int keep_width, keep_ring;
+    int64_t keep_off;       // floats from the slot's start
+    // wkv
+    const float *r, *k, *v, *wraw, *gate;
+    int64_t ld;
+    const float *w0, *u, *norm_w;
+    float eps;
+    void* out;              // wkv: rows in the compute type [n, H * cols]; ssd: float [n, ldy]
+    // ssd
+    const float* xbc;       // [n, ldx]: x at 0, B at inner, C at inner + G * rows
+    int64_t ldx;
+    const float* dtraw;     // [n, ldp], one a head
+    int64_t ldp;
+    const float *dt_bias, *A_log, *Dskip;
+    int64_t ldy;
+    int G, inner;
+};
+
+template <int MODE, int REG, typename OutT>
+__global__ void __launch_bounds__(SCAN_THREADS)
+scan_kernel(ScanArgs a) {
+    extern __shared__ float lds[];
+    const int s = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+    const int R = a.rows, C = a.cols, CL = a.col_lanes;
+    const int n_rb = SCAN_THREADS / CL;
+    const int Rp = n_rb * a.rows_per;  // rows as staged: zeros behind the last
+    float* decay = lds;                           // [CHUNK][Rp]
+    float* inr = decay + SCAN_CHUNK * Rp;         // [CHUNK][Rp]
+    float* qr = inr + SCAN_CHUNK * Rp;            // [CHUNK][Rp]
+    float* val = qr + SCAN_CHUNK * Rp;            // [CHUNK][CL]
+    float* part = val + SCAN_CHUNK * CL;          // [CHUNK][n_rb][CL]
+    float* bonus = part + SCAN_CHUNK * SCAN_THREADS;  // [Rp] (wkv)
+
+    const int begin = a.seq_starts[s], end = a.seq_starts[s + 1];
+    const int slot = a.state_slots[s];
+    const bool slot_ok = slot >= 0 && slot < a.n_slots;
+    const int j = tid % CL, rb = tid / CL;
+    const int i0 = rb * a.rows_per;
+    float* S_glob = a.state + static_cast<int64_t>(slot_ok ? slot : 0) * a.state_stride + static_cast<int64_t>(h) * R * C;
+    const bool fresh = a.positions[begin] == 0;
+
+    float S[REG];
+#pragma unroll
+    for (int ii = 0; ii < REG; ++ii) {
+        const int i = i0 + ii;
+        S[ii] = (ii < a.rows_per && i < R && j < C && slot_ok && !fresh) ? S_glob[static_cast<int64_t>(i) * C + j] : 0.0f;
+    }
+    if (MODE == 0) {
+        for (int i = tid; i < Rp; i += SCAN_THREADS) bonus[i] = i < R ? a.u[h * R + i] : 0.0f;
+    }
+    const int g = MODE == 1 ? h / (a.H / a.G) : 0;
+    const float neg_A = MODE == 1 ? -expf(a.A_log[h]) : 0.0f;
+    const float dskip = MODE == 1 ? a.Dskip[h] : 0.0f;
+
+    for (int c0 = begin; c0 < end; c0 += SCAN_CHUNK) {
+        const int len = min(SCAN_CHUNK, end - c0);
+        __syncthreads();  // the chunk before has been read
+        for (int e = tid; e < len * Rp; e += SCAN_THREADS) {
+            const int tt = e / Rp, i = e % Rp;
+            const int64_t t = c0 + tt;
+            float d = 0.0f, x = 0.0f, q = 0.0f;
+            if (i < R) {
+                if (MODE == 0) {
+                    const int64_t at = t * a.ld + h * R + i;
+                    d = expf(-expf(a.wraw[at] + a.w0[h * R + i]));
+                    x = a.k[at];
+                    q = a.r[at];
+                } else {
+                    const float dt = softplus_f(a.dtraw[t * a.ldp + h] + a.dt_bias[h]);
+                    d = expf(neg_A * dt);
+                    x = dt * a.xbc[t * a.ldx + a.inner + g * R + i];
+                    q = a.xbc[t * a.ldx + a.inner + a.G * R + g * R + i];
+                }
+            }
+            decay[e] = d;
+            inr[e] = x;
+            qr[e] = q;
+        }
+        for (int e = tid; e < len * CL; e += SCAN_THREADS) {
+            const int tt = e / CL, jj = e % CL;
+            const int64_t t = c0 + tt;
+            float x = 0.0f;
+            if (jj < C) x = MODE == 0 ? a.v[t * a.ld + h * C + jj] : a.xbc[t * a.ldx + h * C + jj];
+            val[e] = x;
+        }
+        __syncthreads();
+        for (int tt = 0; tt < len; ++tt) {
+            const float vj = val[tt * CL + j];
+            const float* dr = decay + tt * Rp + i0;
+            const float* ir = inr + tt * Rp + i0;
+            const float* qq = qr + tt * Rp + i0;
+            float acc = 0.0f;
+#pragma unroll
+            for (int ii = 0; ii < REG; ++ii) {
+                if (ii < a.rows_per) {
+                    const float kin = ir[ii] * vj;
+                    if (MODE == 0) {
+                        acc = fmaf(qq[ii], fmaf(bonus[i0 + ii], kin, S[ii]), acc);
+                        S[ii] = fmaf(dr[ii], S[ii], kin);
+                    } else {
+                        S[ii] = fmaf(dr[ii], S[ii], kin);
+                        acc = fmaf(qq[ii], S[ii], acc);
+                    }
+                }
+            }
+            part[(tt * n_rb + rb) * CL + j] = acc;
+        }
+        __syncthreads();
+        if (MODE == 0) {
+            // a wave a token: the head's outputs, their root mean square, the weight and the gate
+            const int wave = tid / kWave, lane = tid % kWave;
+            for (int tt = wave; tt < len; tt += SCAN_THREADS / kWave) {
+                const int64_t t = c0 + tt;
+                float ss = 0.0f;
+                for (int jj = lane; jj < C; jj += kWave) {
+                    float o = 0.0f;
+                    for (int b = 0; b < n_rb; ++b) o += part[(tt * n_rb + b) * CL + jj];
+                    ss = fmaf(o, o, ss);
+                }
+                const float rinv = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(C) + a.eps);
+                for (int jj = lane; jj < C; jj += kWave) {
+                    float o = 0.0f;
+                    for (int b = 0; b < n_rb; ++b) o += part[(tt * n_rb + b) * CL + jj];
+                    const int col = h * C + jj;
+                    const float y = o * rinv * a.norm_w[col] * silu_f(a.gate[t * a.ld + col]);
+                    static_cast<OutT*>(a.out)[t * (static_cast<int64_t>(a.H) * C) + col] = from_float<OutT>(y);
+                }
+            }
+        } else {
+            for (int e = tid; e < len * C; e += SCAN_THREADS) {
+                const int tt = e / C, jj = e % C;
+                float o = 0.0f;
+                for (int b = 0; b < n_rb; ++b) o += part[(tt * n_rb + b) * CL + jj];
+                static_cast<float*>(a.out)[(c0 + tt) * a.ldy + h * C + jj] = fmaf(dskip, val[tt * CL + jj], o);
+            }
+        }
+    }
+    if (slot_ok) {
+#pragma unroll
+        for (int ii = 0; ii < REG; ++ii) {
+            const int i = i0 + ii;
+            if (ii < a.rows_per && i < R && j < C) S_glob[static_cast<int64_t>(i) * C + j] = S[ii];
+        }
+        if (h == 0 && a.keep_src != nullptr && a.keep_ring > 0) {
+            float* dst = a.state + static_cast<int64_t>(slot) * a.state_stride + a.keep_off;
+            const int first = max(begin, end - a.keep_ring);
+            for (int t = first; t < end; ++t) {
+                const int place = a.positions[t] % a.keep_ring;
+                for (int c = tid; c < a.keep_width; c += SCAN_THREADS) {
+                    const int64_t at = static_cast<int64_t>(t) * a.keep_ld + c;
+                    dst[static_cast<int64_t>(place) * a.keep_width + c] =
+                        a.keep_bf16 ? bf16_to_float(static_cast<const bf16_t*>(a.keep_src)[at]) : static_cast<const float*>(a.keep_src)[at];
+                }
+            }
+        }
+    }
+}
+
+// rows a thread holds, lanes side by side, and the dynamic LDS for a state of rows x cols; false when
+// the kernel does not take the size
+static bool scan_shape(int rows, int cols, int* col_lanes, int* rows_per, int* reg, size_t* smem) {
+    if (rows <= 0 || cols <= 0 || cols > SCAN_THREADS) return false;
+    int cl = 1;
+    while (cl < cols) cl *= 2;
+    const int n_rb = SCAN_THREADS / cl;
+    const int rp = (rows + n_rb - 1) / n_rb;
+    if (rp > 64) return false;
+    *col_lanes = cl;
+    *rows_per = rp;
+    *reg = rp <= 8 ? 8 : rp <= 16 ? 16 : rp <= 32 ? 32 : 64;
+    const int Rp = n_rb * rp;
+    *smem = sizeof(float) * (static_cast<size_t>(3) * SCAN_CHUNK * Rp + SCAN_CHUNK * cl + SCAN_CHUNK * SCAN_THREADS + Rp);
+    return *smem <= 64 * 1024;
+}
+
+template <int MODE, typename OutT>
+static void launch_scan(const ScanArgs& a, int n_seqs, int reg, size_t smem, hipStream_t stream) {
+    dim3 grid(n_seqs, a.H);
+    switch (reg) {
+        case 8: scan_kernel<MODE, 8, OutT><<<grid, SCAN_THREADS, smem, stream>>>(a); break;
+        case 16: scan_kernel<MODE, 16, OutT><<<grid, SCAN_THREADS, smem, stream>>>(a); break;
+        case 32: scan_kernel<MODE, 32, OutT><<<grid, SCAN_THREADS, smem, stream>>>(a); break;
+        default: scan_kernel<MODE, 64, OutT><<<grid, SCAN_THREADS, smem, stream>>>(a); break;
+    }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+token_shift_kernel(T* __restrict__ out, const T* __restrict__ h, const float* __restrict__ mu, int n_mix, const float* __restrict__ state,
+                   int64_t state_stride, int n_slots, const int* __restrict__ tok_seq, const int* __restrict__ positions,
+                   const int* __restrict__ seq_starts, const int* __restrict__ state_slots, int n, int d) {
+    const int t = blockIdx.x;
+    const int s = tok_seq[t], p = positions[t];
+    const int slot = state_slots[s];
+    const bool from_step = t > seq_starts[s];
+    const bool from_state = !from_step && p > 0 && slot >= 0 && slot < n_slots;
+    const float* prev_state = state + static_cast<int64_t>(from_state ? slot : 0) * state_stride;
+    for (int i = threadIdx.x; i < d; i += 256) {
+        const float cur = to_float<T>(h[static_cast<int64_t>(t) * d + i]);
+        float prev = 0.0f;
+        if (p > 0) prev = from_step ? to_float<T>(h[static_cast<int64_t>(t - 1) * d + i]) : (from_state ? prev_state[i] : 0.0f);
+        const float diff = prev - cur;
+        for (int c = 0; c < n_mix; ++c)
+            out[(static_cast<int64_t>(c) * n + t) * d + i] = from_float<T>(fmaf(diff, mu[c * d + i], cur));
+    }
+}
+
+__global__ void __launch_bounds__(256)
+conv_act_kernel(float* __restrict__ out, int64_t ldo, const float* __restrict__ in, int64_t ldi, const float* __restrict__ w,
+                const float* __restrict__ bias, int taps, const float* __restrict__ state, int64_t state_stride, int n_slots,
+                const int* __restrict__ tok_seq, const int* __restrict__ positions, const int* __restrict__ seq_starts,
+                const int* __restrict__ state_slots, int C) {
+    const int t = blockIdx.y;
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= C) return;
+    const int s = tok_seq[t], p = positions[t];
+    const int begin = seq_starts[s];
+    const int slot = state_slots[s];
+    const bool slot_ok = slot >= 0 && slot < n_slots;
+    const float* ring = state + static_cast<int64_t>(slot_ok ? slot : 0) * state_stride;
+    float acc = bias != nullptr ? bias[c] : 0.0f;
+    for (int jt = 0; jt < taps; ++jt) {
+        const int back = taps - 1 - jt;  // rows before this one
+        const int sp = p - back;
+        if (sp < 0) continue;
+        float x;
+        if (t - back >= begin) x = in[static_cast<int64_t>(t - back) * ldi + c];
+        else x = slot_ok ? ring[static_cast<int64_t>(sp % (taps - 1)) * C + c] : 0.0f;
+        acc = fmaf(w[static_cast<int64_t>(c) * taps + jt], x, acc);
+    }
+    out[static_cast<int64_t>(t) * ldo + c] = silu_f(acc);
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+gated_group_norm_kernel(T* __restrict__ out, const float* __restrict__ y, int64_t ldy, const float* __restrict__ z, int64_t ldz,
+                        const float* __restrict__ w, float eps, int inner, int groups) {
+    __shared__ float red[256 / kWave];
+    const int t = blockIdx.x, g = blockIdx.y;
+    const int width = inner / groups;
+    const float* yr = y + static_cast<int64_t>(t) * ldy + g * width;
+    const float* zr = z + static_cast<int64_t>(t) * ldz + g * width;
+    float ss = 0.0f;
+    for (int i = threadIdx.x; i < width; i += 256) {
+        const float v = yr[i] * silu_f(zr[i]);
+        ss = fmaf(v, v, ss);
+    }
+    ss = wave_sum(ss);
+    if (threadIdx.x % kWave == 0) red[threadIdx.x / kWave] = ss;
+    __syncthreads();
+    float total = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 256 / kWave; ++i) total += red[i];
+    const float rinv = 1.0f / sqrtf(total / static_cast<float>(width) + eps);
+    for (int i = threadIdx.x; i < width; i += 256) {
+        const float v = yr[i] * silu_f(zr[i]) * rinv * w[g * width + i];
+        out[static_cast<int64_t>(t) * inner + g * width + i] = from_float<T>(v);
+    }
+}
+
+}  // namespace liyab
+
+using namespace liyab;
+
+extern "C" int liyab_scan_takes(int rows, int cols) {
+    int cl, rp, reg;
+    size_t smem;
+    return scan_shape(rows, cols, &cl, &rp, &reg, &smem) ? 1 : 0;
+}
+
+extern "C" int liyab_wkv_scan(void* out, int out_dtype, const float* r, const float* k, const float* v, const float* wraw, const float* gate,
+                              int64_t ld, const float* w0, const float* u, const float* norm_w, float eps, float* state, int64_t state_stride,
+                              int n_slots, const void* keep_src, int keep_dtype, int64_t keep_ld, int keep_width, int64_t keep_off,
+                              const int* seq_starts, const int* positions, const int* state_slots, int n_seqs, int H, int D,
+                              hipStream_t stream) {
+    LIYAB_REQUIRE(out && r && k && v && wraw && gate && w0 && u && norm_w && state && seq_starts && positions && state_slots, "wkv_scan: null pointer");
+    LIYAB_REQUIRE(n_seqs >= 0 && H > 0 && D > 0 && n_slots > 0, "wkv_scan: bad sizes");
+    LIYAB_REQUIRE(ld >= static_cast<int64_t>(H) * D, "wkv_scan: rows shorter than heads x head size");
+    LIYAB_REQUIRE(state_stride >= static_cast<int64_t>(H) * D * D + (keep_src ? keep_off - static_cast<int64_t>(H) * D * D + keep_width : 0) &&
+                      (keep_src == nullptr || keep_off >= static_cast<int64_t>(H) * D * D),
+                  "wkv_scan: a slot of %lld floats does not hold the state", static_cast<long long>(state_stride));
+    ScanArgs a = {};
+    size_t smem;
+    int reg;
+    LIYAB_REQUIRE(scan_shape(D, D, &a.col_lanes, &a.rows_per, &reg, &smem), "wkv_scan: heads of %d are not taken", D);
+    if (n_seqs == 0) return 0;
+    a.state = state; a.state_stride = state_stride; a.n_slots = n_slots;
+    a.seq_starts = seq_starts; a.positions = positions; a.state_slots = state_slots;
+    a.H = H; a.rows = D; a.cols = D;
+    a.keep_src = keep_src; a.keep_bf16 = keep_dtype == kBF16; a.keep_ld = keep_ld; a.keep_width = keep_width; a.keep_ring = 1; a.keep_off = keep_off;
+    a.r = r; a.k = k; a.v = v; a.wraw = wraw; a.gate = gate; a.ld = ld; a.w0 = w0; a.u = u; a.norm_w = norm_w; a.eps = eps; a.out = out;
+    if (out_dtype == kF32) launch_scan<0, float>(a, n_seqs, reg, smem, stream);
+    else if (out_dtype == kBF16) launch_scan<0, bf16_t>(a, n_seqs, reg, smem, stream);
+    else return fail(1, "wkv_scan: unknown dtype %d", out_dtype);
+    return check_launch("wkv_scan");
+}
+
+extern "C" int liyab_ssd_scan(float* y, int64_t ldy, const float* xbc, int64_t ldx, const float* dtraw, int64_t ldp, const float* dt_bias,
+                              const float* A_log, const float* Dskip, float* state, int64_t state_stride, int n_slots, const float* keep_src,
+                              int64_t keep_ld, int keep_width, int keep_ring, int64_t keep_off, const int* seq_starts, const int* positions,
+                              const int* state_slots, int n_seqs, int H, int P, int N, int G, hipStream_t stream) {
+    LIYAB_REQUIRE(y && xbc && dtraw && dt_bias && A_log && Dskip && state && seq_starts && positions && state_slots, "ssd_scan: null pointer");
+    LIYAB_REQUIRE(n_seqs >= 0 && H > 0 && P > 0 && N > 0 && G > 0 && H % G == 0 && n_slots > 0, "ssd_scan: bad sizes");
+    const int64_t inner = static_cast<int64_t>(H) * P;
+    LIYAB_REQUIRE(ldy >= inner && ldx >= inner + 2 * static_cast<int64_t>(G) * N && ldp >= H, "ssd_scan: rows shorter than their parts");
+    LIYAB_REQUIRE(state_stride >= inner * N && (keep_src == nullptr || (keep_off >= inner * N && state_stride >= keep_off + static_cast<int64_t>(keep_ring) * keep_width)),
+                  "ssd_scan: a slot of %lld floats does not hold the state", static_cast<long long>(state_stride));
+    ScanArgs a = {};
+    size_t smem;
+    int reg;
+    LIYAB_REQUIRE(scan_shape(N, P, &a.col_lanes, &a.rows_per, &reg, &smem), "ssd_scan: a state of %d x %d a head is not taken", N, P);
+    if (n_seqs == 0) return 0;
+    a.state = state; a.state_stride = state_stride; a.n_slots = n_slots;
+    a.seq_starts = seq_starts; a.positions = positions; a.state_slots = state_slots;
+    a.H = H; a.rows = N; a.cols = P;
+    a.keep_src = keep_src; a.keep_bf16 = 0; a.keep_ld = keep_ld; a.keep_width = keep_width; a.keep_ring = keep_ring; a.keep_off = keep_off;
+    a.out = y; a.ldy = ldy; a.xbc = xbc; a.ldx = ldx; a.dtraw = dtraw; a.ldp = ldp; a.dt_bias = dt_bias; a.A_log = A_log; a.Dskip = Dskip;
+    a.G = G; a.inner = static_cast<int>(inner);
+    launch_scan<1, float>(a, n_seqs, reg, smem, stream);
+    return check_launch("ssd_scan");
+}
+
+extern "C" int liyab_token_shift(void* out, int dtype, const void* h, const float* mu, int n_mix, const float* state, int64_t state_stride,
+                                 int n_slots, const int* tok_seq, const int* positions, const int* seq_starts, const int* state_slots, int n,
+                                 int d, hipStream_t stream) {
+    LIYAB_REQUIRE(out && h && mu && state && tok_seq && positions && seq_starts && state_slots, "token_shift: null pointer");
+    LIYAB_REQUIRE(n >= 0 && d > 0 && n_mix > 0 && n_slots > 0 && state_stride >= d, "token_shift: bad sizes");
+    if (n == 0) return 0;
+    if (dtype == kF32)
+        token_shift_kernel<float><<<n, 256, 0, stream>>>(static_cast<float*>(out), static_cast<const float*>(h), mu, n_mix, state, state_stride,
+                                                          n_slots, tok_seq, positions, seq_starts, state_slots, n, d);
+    else if (dtype == kBF16)
+        token_shift_kernel<bf16_t><<<n, 256, 0, stream>>>(static_cast<bf16_t*>(out), static_cast<const bf16_t*>(h), mu, n_mix, state, state_stride,
+                                                           n_slots, tok_seq, positions, seq_starts, state_slots, n, d);
+    else return fail(1, "token_shift: unknown dtype %d", dtype);
+    return check_launch("token_shift");
+}
+
+extern "C" int liyab_conv_act(float* out, int64_t ldo, const float* in, int64_t ldi, const float* w, const float* bias, int taps,
+                              const float* state, int64_t state_stride, int n_slots, const int* tok_seq, const int* positions,
+                              const int* seq_starts, const int* state_slots, int n, int C, hipStream_t stream) {
+    LIYAB_REQUIRE(out && in && w && tok_seq && positions && seq_starts && state_slots, "conv_act: null pointer");
+    LIYAB_REQUIRE(n >= 0 && n <= 65535 && C > 0 && taps >= 1 && ldo >= C && ldi >= C, "conv_act: bad sizes");
+    LIYAB_REQUIRE(taps == 1 || (state != nullptr && n_slots > 0 && state_stride >= static_cast<int64_t>(taps - 1) * C),
+                  "conv_act: %d taps need the last %d rows of a request in its slot", taps, taps - 1);
+    if (n == 0) return 0;
+    dim3 grid((C + 255) / 256, n);
+    conv_act_kernel<<<grid, 256, 0, stream>>>(out, ldo, in, ldi, w, bias, taps, state, state_stride, taps > 1 ? n_slots : 0, tok_seq, positions,
+                                              seq_starts, state_slots, C);
+    return check_launch("conv_act");
+}
+
+extern "C" int liyab_gated_group_norm(void* out, int out_dtype, const float* y, int64_t ldy, const float* z, int64_t ldz, const float* w,
+                                      float eps, int n, int inner, int groups, hipStream_t stream) {
+    LIYAB_REQUIRE(out && y && z && w, "gated_group_norm: null pointer");
+    LIYAB_REQUIRE(n >= 0 && inner > 0 && groups > 0 && groups <= 65535 && inner % groups == 0 && ldy >= inner && ldz >= inner, "gated_group_norm: bad sizes");
+    if (n == 0) return 0;
+    dim3 grid(n, groups);
+    if (out_dtype == kF32) gated_group_norm_kernel<float><<<grid, 256, 0, stream>>>(static_cast<float*>(out), y, ldy, z, ldz, w, eps, inner, groups);
+    else if (out_dtype == kBF16) gated_group_norm_kernel<bf16_t><<<grid, 256, 0, stream>>>(static_cast<bf16_t*>(out), y, ldy, z, ldz, w, eps, inner, groups);
+    else return fail(1, "gated_group_norm: unknown dtype %d", out_dtype);
+    return check_launch("gated_group_norm");
+}

@@ -96,6 +96,17 @@ static const Entry kEntries[] = {
     LIYAB_ENTRY(liyab_moe_route),
     LIYAB_ENTRY(liyab_moe_align),
     LIYAB_ENTRY(liyab_moe_route_align),
+    LIYAB_ENTRY(liyab_dyt),
+    LIYAB_ENTRY(liyab_glu_clamped),
+    LIYAB_ENTRY(liyab_activate),
+    LIYAB_ENTRY(liyab_mean_norm_add),
+    LIYAB_ENTRY(liyab_wkv_scan),
+    LIYAB_ENTRY(liyab_ssd_scan),
+    LIYAB_ENTRY(liyab_token_shift),
+    LIYAB_ENTRY(liyab_conv_act),
+    LIYAB_ENTRY(liyab_gated_group_norm),
+    LIYAB_ENTRY(liyab_qk_prepare),
+    LIYAB_ENTRY(liyab_attention_scored),
 };
 constexpr int kNumEntries = static_cast<int>(sizeof(kEntries) / sizeof(kEntries[0]));
 

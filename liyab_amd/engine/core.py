@@ -57,6 +57,8 @@ class EngineCore:
                 num_pages = -(-max_tokens // page_size)
             else:
                 num_pages = max_requests * (-(-max_positions // page_size))
+        # no request holds more positions than the pool has: block tables are no wider than that
+        max_positions = min(max_positions, max(1, num_pages) * page_size)
         self.manager = CacheManager(self.model.cache_groups(), page_size=page_size, num_pages=max(1, num_pages),
                                     max_requests=max_requests, max_positions=max_positions)
         self.storage = CacheStorage(self.manager, self.dtype, self.device, self.model.state_specs())

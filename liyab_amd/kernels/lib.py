@@ -82,6 +82,21 @@ _SIGNATURES = {
     "liyab_moe_route": [P, c_int64, c_int, c_int, c_int, P, P, P],
     "liyab_moe_align": [P, c_int, c_int, c_int, P, P, c_int, P],
     "liyab_moe_route_align": [P, c_int64, c_int, c_int, c_int, P, P, c_int, P, P, c_int, P],
+    "liyab_dyt": [P, c_int, P, P, P, P, P, c_int, c_int, P],
+    "liyab_glu_clamped": [P, c_int, P, c_int64, c_int, c_int, c_float, c_float, c_float, P],
+    "liyab_activate": [P, c_int, c_int64, P, c_int64, c_int, c_int, c_int, P],
+    "liyab_mean_norm_add": [P, P, P, P, P, c_float, c_float, c_int, c_int, P],
+    "liyab_wkv_scan": [P, c_int, P, P, P, P, P, c_int64, P, P, P, c_float, P, c_int64, c_int, P, c_int, c_int64, c_int, c_int64, P, P, P,
+                       c_int, c_int, c_int, P],
+    "liyab_ssd_scan": [P, c_int64, P, c_int64, P, c_int64, P, P, P, P, c_int64, c_int, P, c_int64, c_int, c_int, c_int64, P, P, P, c_int,
+                       c_int, c_int, c_int, c_int, P],
+    "liyab_token_shift": [P, c_int, P, P, c_int, P, c_int64, c_int, P, P, P, P, c_int, c_int, P],
+    "liyab_conv_act": [P, c_int64, P, c_int64, P, P, c_int, P, c_int64, c_int, P, P, P, P, c_int, c_int, P],
+    "liyab_gated_group_norm": [P, c_int, P, c_int64, P, c_int64, P, c_float, c_int, c_int, c_int, P],
+    "liyab_qk_prepare": [P, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P, P, P, c_int, P, c_int, c_int, P, P, c_float, P,
+                         c_int, c_float, c_int, P, c_int, P],
+    "liyab_attention_scored": [P, c_int64, P, c_int64, P, P, c_int, P, c_int, P, P, c_int, c_float, c_float, c_int, P, c_int, P, c_int64,
+                               c_int, c_int, c_int, c_int, c_int, c_int, P],
 }
 
 
@@ -121,7 +136,8 @@ def load() -> ctypes.CDLL:
         fn.restype = c_int
         fn.argtypes = args
     for name, args in (("liyab_replay_index", [c_char_p, ctypes.POINTER(c_int)]),
-                       ("liyab_replay", [ctypes.POINTER(ctypes.c_uint64), c_int64])):
+                       ("liyab_replay", [ctypes.POINTER(ctypes.c_uint64), c_int64]),
+                       ("liyab_scan_takes", [c_int, c_int])):
         fn = getattr(lib, name, None)
         if fn is None:
             raise KernelError(f"'{path}' lacks the entry point {name}: rebuild it (python -m liyab_amd.csrc.build)")

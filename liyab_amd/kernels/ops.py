@@ -1241,3 +1241,282 @@ def moe_product(out: torch.Tensor, a: torch.Tensor, w0: torch.Tensor, w1: Option
     _lib.call("liyab_grouped_product", a.data_ptr(), lda, a_div, 0, w0.data_ptr(), _ptr(w1), dtype_code(a.dtype), out.data_ptr(),
               dtype_code(out.dtype), ldo, 0, rows_list.data_ptr(), tile_group.data_ptr(), tiles, block, E, _ptr(row_scale), None, F32, 0,
               entries, N, K, _stream())
+
+
+# -- norms without statistics, clamped gated activations, two sublayers' results joined ------------
+def dyt(out: torch.Tensor, x: torch.Tensor, weight: Optional[torch.Tensor], bias: Optional[torch.Tensor], alpha: torch.Tensor,
+        rows: Optional[torch.Tensor] = None) -> None:
+    """out[r] = tanh(alpha * x[rows[r]] (or x[r])) * weight + bias; x float32 [*, d], alpha one float32 value on the
+    device, out [n, d] float32 or bfloat16."""
+    _dev(out, "out")
+    _dev(x, "x")
+    n, d = out.shape
+    if x.dtype != torch.float32 or x.dim() != 2 or x.shape[1] != d or not x.is_contiguous() or not out.is_contiguous():
+        raise KernelError(f"dyt: x must be contiguous float32 [*, {d}] and out contiguous, got {tuple(x.shape)} {x.dtype}")
+    _f32vec(weight, "norm weight", d)
+    _f32vec(bias, "norm bias", d)
+    _f32vec(alpha, "norm alpha", 1)
+    if rows is not None:
+        _i32(rows, "rows", n)
+    elif x.shape[0] < n:
+        raise KernelError("dyt: fewer input rows than output rows")
+    _lib.call("liyab_dyt", out.data_ptr(), dtype_code(out.dtype), x.data_ptr(), _ptr(weight), _ptr(bias), alpha.data_ptr(), _ptr(rows), n, d, _stream())
+
+
+def glu_clamped(out: torch.Tensor, gu: torch.Tensor, limit: float, slope: float, shift: float) -> None:
+    """out = g * sigmoid(slope * g) * (u + shift) with g = min(G, limit), u = clamp(U, -limit, limit); gu float32
+    [n, 2 * ff] = [G | U], out contiguous [n, ff] float32 or bfloat16."""
+    _dev(out, "out")
+    ld = _rows(gu, "gu")
+    n, ff = out.shape
+    if gu.dtype != torch.float32 or tuple(gu.shape) != (n, 2 * ff) or not out.is_contiguous():
+        raise KernelError(f"glu_clamped: needs float32 [n, {2 * ff}] and a contiguous out [n, {ff}], got {tuple(gu.shape)} {gu.dtype}")
+    _lib.call("liyab_glu_clamped", out.data_ptr(), dtype_code(out.dtype), gu.data_ptr(), ld, n, ff, float(limit), float(slope), float(shift), _stream())
+
+
+ACTIVATE = {"tanh": 0, "silu": 1, "sigmoid": 2}
+
+
+def activate(out: torch.Tensor, x: torch.Tensor, op: str) -> None:
+    """out = op(x), x float32 rows, out rows of the same shape in float32 or bfloat16."""
+    ldo, ldi = _rows(out, "out"), _rows(x, "x")
+    if x.dtype != torch.float32 or out.shape != x.shape:
+        raise KernelError("activate: x must be float32 and out of its shape")
+    _lib.call("liyab_activate", out.data_ptr(), dtype_code(out.dtype), ldo, x.data_ptr(), ldi, ACTIVATE[op], x.shape[0], x.shape[1], _stream())
+
+
+def mean_norm_add(x: torch.Tensor, a: torch.Tensor, b: torch.Tensor, wa: torch.Tensor, wb: torch.Tensor, eps: float, weight: float = 0.5) -> None:
+    """x += weight * (a / rms(a) * wa + b / rms(b) * wb), all float32 [n, d] contiguous, rms over a row with eps inside the root."""
+    n, d = x.shape
+    for t, what in ((x, "x"), (a, "a"), (b, "b")):
+        _dev(t, what)
+        if t.dtype != torch.float32 or tuple(t.shape) != (n, d) or not t.is_contiguous():
+            raise KernelError(f"mean_norm_add: {what} must be contiguous float32 [{n}, {d}]")
+    _f32vec(wa, "weight a", d)
+    _f32vec(wb, "weight b", d)
+    _lib.call("liyab_mean_norm_add", x.data_ptr(), a.data_ptr(), b.data_ptr(), wa.data_ptr(), wb.data_ptr(), float(eps), float(weight), n, d, _stream())
+
+
+# -- mixers with a matrix of state a head ---------------------------------------------------------------
+def scan_takes(rows: int, cols: int) -> bool:
+    """Whether the recurrence kernel takes a state of rows x cols a head (csrc/recurrent.hip: scan_shape): a column a
+    thread, up to 64 rows of it in registers, sixteen tokens' vectors staged in at most 64 KiB of LDS."""
+    if rows <= 0 or not 0 < cols <= 256:
+        return False
+    lanes = 1
+    while lanes < cols:
+        lanes *= 2
+    blocks = 256 // lanes
+    per = -(-rows // blocks)
+    staged = blocks * per
+    return per <= 64 and 4 * (3 * 16 * staged + 16 * lanes + 16 * 256 + staged) <= 64 * 1024
+
+
+def _step_lists(ctx, n: int) -> None:
+    _i32(ctx.tok_seq, "tok_seq", n)
+    _i32(ctx.positions, "positions", n)
+    _i32(ctx.seq_starts, "seq_starts", ctx.n_seqs + 1)
+    _i32(ctx.state_slots, "state_slots", ctx.n_seqs)
+
+
+def _state(state: torch.Tensor, what: str) -> int:
+    _dev(state, "state")
+    if state.dtype != torch.float32 or state.dim() != 2 or not state.is_contiguous():
+        raise KernelError(f"{what}: the state must be contiguous float32 [slots, floats a slot], got {tuple(state.shape)} {state.dtype}")
+    return state.shape[1]
+
+
+def token_shift(out: torch.Tensor, h: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, prev_off: int, ctx) -> None:
+    """out[c, t] = h[t] + (h[t - 1] - h[t]) * mu[c]; h [n, d] in the compute dtype, mu float32 [n_mix, d], out [n_mix, n, d];
+    the row before a request's first row of the step is state[slot, prev_off : prev_off + d], zeros at position 0."""
+    _dev(out, "out")
+    _dev(h, "h")
+    n, d = h.shape
+    stride = _state(state, "token_shift")
+    if not h.is_contiguous() or not out.is_contiguous() or out.dtype != h.dtype or mu.dim() != 2 or tuple(out.shape) != (mu.shape[0], n, d):
+        raise KernelError("token_shift: h [n, d] and out [n_mix, n, d] must be contiguous and of one dtype")
+    _f32vec(mu, "mu", mu.shape[0] * d)
+    if prev_off < 0 or prev_off + d > stride or ctx.n_tokens != n:
+        raise KernelError("token_shift: the previous row does not lie in the slot, or h is not the step's rows")
+    _step_lists(ctx, n)
+    _lib.call("liyab_token_shift", out.data_ptr(), dtype_code(h.dtype), h.data_ptr(), mu.data_ptr(), mu.shape[0], state.data_ptr() + 4 * prev_off,
+              stride, state.shape[0], ctx.tok_seq.data_ptr(), ctx.positions.data_ptr(), ctx.seq_starts.data_ptr(), ctx.state_slots.data_ptr(),
+              n, d, _stream())
+
+
+def wkv_scan(out: torch.Tensor, proj: torch.Tensor, w0: torch.Tensor, u: torch.Tensor, norm_w: torch.Tensor, eps: float, state: torch.Tensor,
+             h: torch.Tensor, ctx, *, n_head: int, head_dim: int) -> None:
+    """The decayed outer-product recurrence with a bonus over each request's rows of the step. proj float32 [n, 5 * H * D] =
+    [r | k | v | gate logits | raw decay]; decay = exp(-exp(raw + w0)); per head o = (S + diag(u) k v^T)^T r, S <- diag(decay) S
+    + k v^T; out [n, H * D] (compute dtype) = o / rms(o over the head) * norm_w * silu(gate). state float32 [slots, H * D * D + width]:
+    the heads' matrices, then the request's last row of h [n, width], which is kept here for the next step's token shift."""
+    _dev(out, "out")
+    n, HD = out.shape
+    H, D = n_head, head_dim
+    stride = _state(state, "wkv_scan")
+    ld = _rows(proj, "proj")
+    if HD != H * D or proj.dtype != torch.float32 or tuple(proj.shape) != (n, 5 * HD) or not out.is_contiguous():
+        raise KernelError(f"wkv_scan: needs float32 proj [n, {5 * H * D}] and a contiguous out [n, {H * D}], got {tuple(proj.shape)} {proj.dtype}")
+    for t, what in ((w0, "w0"), (u, "u"), (norm_w, "norm weight")):
+        _f32vec(t, what, HD)
+    _dev(h, "h")
+    if h.dim() != 2 or h.shape[0] != n or not h.is_contiguous() or stride != H * D * D + h.shape[1] or ctx.n_tokens != n:
+        raise KernelError("wkv_scan: the state must hold the heads' matrices and one row of h")
+    if not scan_takes(D, D):
+        raise KernelError(f"wkv_scan: heads of {D} are not taken")
+    _step_lists(ctx, n)
+    p = proj.data_ptr()
+    _lib.call("liyab_wkv_scan", out.data_ptr(), dtype_code(out.dtype), p, p + 4 * HD, p + 8 * HD, p + 16 * HD, p + 12 * HD, ld, w0.data_ptr(),
+              u.data_ptr(), norm_w.data_ptr(), float(eps), state.data_ptr(), stride, state.shape[0], h.data_ptr(), dtype_code(h.dtype),
+              h.shape[1], h.shape[1], H * D * D, ctx.seq_starts.data_ptr(), ctx.positions.data_ptr(), ctx.state_slots.data_ptr(), ctx.n_seqs,
+              H, D, _stream())
+
+
+def conv_act(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], state: Optional[torch.Tensor],
+             ring_off: int, ctx) -> None:
+    """out[t, c] = silu(bias[c] + sum_j weight[c, j] * x[t - taps + 1 + j, c]) over each request's own rows in time; x, out float32
+    rows (columns of wider rows are fine), weight float32 [C, taps]; the rows before a request's first row of the step come from
+    state[slot, ring_off + (position % (taps - 1)) * C + c], zeros before position 0."""
+    ldo, ldi = _rows(out, "out"), _rows(x, "x")
+    n, C = x.shape
+    if x.dtype != torch.float32 or out.dtype != torch.float32 or tuple(out.shape) != (n, C) or ctx.n_tokens != n:
+        raise KernelError("conv_act: x and out must be the step's float32 rows of one shape")
+    _dev(weight, "weight")
+    if weight.dtype != torch.float32 or weight.dim() != 2 or weight.shape[0] != C or not weight.is_contiguous():
+        raise KernelError(f"conv_act: the weight must be contiguous float32 [{C}, taps]")
+    taps = weight.shape[1]
+    _f32vec(bias, "bias", C)
+    stride, slots, base = 0, 0, None
+    if taps > 1:
+        stride = _state(state, "conv_act")
+        if ring_off < 0 or ring_off + (taps - 1) * C > stride:
+            raise KernelError("conv_act: the ring does not lie in the slot")
+        slots, base = state.shape[0], state.data_ptr() + 4 * ring_off
+    _step_lists(ctx, n)
+    _lib.call("liyab_conv_act", out.data_ptr(), ldo, x.data_ptr(), ldi, weight.data_ptr(), _ptr(bias), taps, base, stride, slots,
+              ctx.tok_seq.data_ptr(), ctx.positions.data_ptr(), ctx.seq_starts.data_ptr(), ctx.state_slots.data_ptr(), n, C, _stream())
+
+
+def ssd_scan(y: torch.Tensor, xbc: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor, d_skip: torch.Tensor,
+             state: torch.Tensor, keep_src: Optional[torch.Tensor], keep_ring: int, ctx, *, n_head: int, head_dim: int, n_state: int,
+             n_groups: int) -> None:
+    """The selective state-space recurrence over each request's rows of the step: dt = softplus(dt_raw + dt_bias), per head
+    S <- exp(-exp(a_log) dt) S + dt B x^T, y = S^T C + d_skip x. xbc float32 [n, inner + 2 * groups * state] = [x | B | C],
+    dt_raw float32 [n, heads] (columns of wider rows are fine), y float32 [n, inner]. state float32 [slots, inner * state +
+    keep_ring * channels]: the heads' matrices, then the last `keep_ring` rows of keep_src [n, channels] at ring place position %
+    keep_ring, which are kept here for the next step's convolution."""
+    H, P, N, G = n_head, head_dim, n_state, n_groups
+    inner = H * P
+    n = y.shape[0]
+    ldy, ldx, ldp = _rows(y, "y"), _rows(xbc, "xbc"), _rows(dt_raw, "dt_raw")
+    stride = _state(state, "ssd_scan")
+    if (y.dtype != torch.float32 or xbc.dtype != torch.float32 or dt_raw.dtype != torch.float32 or tuple(y.shape) != (n, inner)
+            or tuple(xbc.shape) != (n, inner + 2 * G * N) or tuple(dt_raw.shape) != (n, H) or ctx.n_tokens != n):
+        raise KernelError("ssd_scan: y [n, inner], xbc [n, inner + 2 groups x state] and dt_raw [n, heads] must be the step's float32 rows")
+    for t, what in ((dt_bias, "dt_bias"), (a_log, "A_log"), (d_skip, "D")):
+        _f32vec(t, what, H)
+    kptr, kld, kw = None, 0, 0
+    if keep_src is not None and keep_ring > 0:
+        kld = _rows(keep_src, "keep_src")
+        kw = keep_src.shape[1]
+        if keep_src.dtype != torch.float32 or keep_src.shape[0] != n:
+            raise KernelError("ssd_scan: the kept rows must be the step's float32 rows")
+        kptr = keep_src.data_ptr()
+    if stride != inner * N + (keep_ring * kw if kptr is not None else 0):
+        raise KernelError("ssd_scan: the state must hold the heads' matrices and the kept rows")
+    if not scan_takes(N, P):
+        raise KernelError(f"ssd_scan: a state of {N} x {P} a head is not taken")
+    _step_lists(ctx, n)
+    _lib.call("liyab_ssd_scan", y.data_ptr(), ldy, xbc.data_ptr(), ldx, dt_raw.data_ptr(), ldp, dt_bias.data_ptr(), a_log.data_ptr(),
+              d_skip.data_ptr(), state.data_ptr(), stride, state.shape[0], kptr, kld, kw, keep_ring if kptr is not None else 0, inner * N,
+              ctx.seq_starts.data_ptr(), ctx.positions.data_ptr(), ctx.state_slots.data_ptr(), ctx.n_seqs, H, P, N, G, _stream())
+
+
+def gated_group_norm(out: torch.Tensor, y: torch.Tensor, z: torch.Tensor, weight: torch.Tensor, eps: float, groups: int) -> None:
+    """out = (y * silu(z)) / rms(.) * weight, the root mean square over each of `groups` equal parts of a row; y, z float32 rows
+    [n, inner] (columns of wider rows are fine), out contiguous [n, inner] float32 or bfloat16."""
+    _dev(out, "out")
+    ldy, ldz = _rows(y, "y"), _rows(z, "z")
+    n, inner = out.shape
+    if y.dtype != torch.float32 or z.dtype != torch.float32 or tuple(y.shape) != (n, inner) or tuple(z.shape) != (n, inner) or not out.is_contiguous():
+        raise KernelError("gated_group_norm: y and z must be float32 [n, inner], out contiguous [n, inner]")
+    if groups < 1 or inner % groups != 0:
+        raise KernelError(f"gated_group_norm: {inner} channels in {groups} parts")
+    _f32vec(weight, "norm weight", inner)
+    _lib.call("liyab_gated_group_norm", out.data_ptr(), dtype_code(out.dtype), y.data_ptr(), ldy, z.data_ptr(), ldz, weight.data_ptr(), float(eps),
+              n, inner, groups, _stream())
+
+
+# -- attention whose scores are more than scale * q . k ---------------------------------------------------
+def qk_prepare(src: torch.Tensor, q_out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, slots: torch.Tensor, positions: torch.Tensor,
+               *, q_off: int, k_off: int, v_off: int, n_head: int, q_norm: Optional[torch.Tensor] = None, k_norm: Optional[torch.Tensor] = None,
+               eps: float = 0.0, freqs: Optional[torch.Tensor] = None, rot_dims: int = 0, temp_coef: float = 0.0, temp_every: int = 0,
+               num_pages: Optional[int] = None) -> None:
+    """From a projection's float32 rows `src` (queries at column q_off, keys at k_off, values at v_off, which may be k_off) to
+    queries in `q_out` [n, heads * dk] and keys and values in their slots of the pages (k_cache [pages, kv_heads, page, dk],
+    v_cache [.., dv]), all in the compute dtype. Per head, each optional: a root-mean-square norm with a weight [dk] (queries,
+    keys), pairs (2i, 2i + 1) of the first rot_dims entries turned by position * freqs[i] (queries, keys), the query times
+    1 + temp_coef * ln(floor((position + 1) / temp_every) + 1). A slot outside the pages is not written."""
+    ld = _rows(src, "src")
+    n = src.shape[0]
+    _dev(q_out, "q_out")
+    _dev(k_cache, "k_cache")
+    _dev(v_cache, "v_cache")
+    if k_cache.dim() != 4 or v_cache.dim() != 4 or k_cache.shape[:3] != v_cache.shape[:3] or not k_cache.is_contiguous() or not v_cache.is_contiguous():
+        raise KernelError("qk_prepare: caches must be contiguous [pages, kv_heads, page_size, width] with the same pages")
+    _, G, page, dk = k_cache.shape
+    dv = v_cache.shape[3]
+    if src.dtype != torch.float32 or tuple(q_out.shape) != (n, n_head * dk) or not q_out.is_contiguous() or not (q_out.dtype == k_cache.dtype == v_cache.dtype):
+        raise KernelError("qk_prepare: src must be float32 rows, q_out contiguous [n, heads * dk], queries and caches of one dtype")
+    if min(q_off, k_off, v_off) < 0 or q_off + n_head * dk > src.shape[1] or k_off + G * dk > src.shape[1] or v_off + G * dv > src.shape[1]:
+        raise KernelError("qk_prepare: the heads' columns pass the source's rows")
+    _f32vec(q_norm, "query norm weight", dk)
+    _f32vec(k_norm, "key norm weight", dk)
+    if rot_dims:
+        if rot_dims % 2 or rot_dims > dk or freqs is None:
+            raise KernelError(f"qk_prepare: {rot_dims} turned entries of heads of {dk}")
+        _f32vec(freqs, "freqs", rot_dims // 2)
+    _i32(slots, "slots", n)
+    _i32(positions, "positions", n)
+    _lib.call("liyab_qk_prepare", src.data_ptr(), ld, q_off, k_off, v_off, n_head, G, dk, dv, q_out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+              dtype_code(q_out.dtype), slots.data_ptr(), page, _pages(k_cache, num_pages), _ptr(q_norm), _ptr(k_norm), float(eps),
+              _ptr(freqs) if rot_dims else None, rot_dims, float(temp_coef), int(temp_every), positions.data_ptr(), n, _stream())
+
+
+def attention_scored(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor, ctx, *,
+                     n_head: int, scale: float, softcap: float = 0.0, window: int = 0, bias_table: Optional[torch.Tensor] = None,
+                     gate: Optional[torch.Tensor] = None, num_pages: Optional[int] = None) -> None:
+    """Causal attention of the step's rows over their requests' pages with score = scale * q . k, then cap * tanh(score / cap)
+    (softcap > 0), then + bias_table[min(distance, rows - 1), head] (float32 [rows, heads]); softmax in 32-bit; values `dv` wide.
+    out [n, heads * dv] = result * sigmoid(gate) (gate: float32 rows [n, heads * dv], or None)."""
+    _dev(out, "out")
+    _dev(q, "q")
+    n = out.shape[0]
+    if k_cache.dim() != 4 or v_cache.dim() != 4 or k_cache.shape[:3] != v_cache.shape[:3] or not k_cache.is_contiguous() or not v_cache.is_contiguous():
+        raise KernelError("attention_scored: caches must be contiguous [pages, kv_heads, page_size, width] with the same pages")
+    _, G, page, dk = k_cache.shape
+    dv = v_cache.shape[3]
+    so, sq = _rows(out, "out"), _rows(q, "q")
+    if tuple(q.shape) != (n, n_head * dk) or tuple(out.shape) != (n, n_head * dv) or not (q.dtype == out.dtype == k_cache.dtype == v_cache.dtype):
+        raise KernelError("attention_scored: q [n, heads * dk], out [n, heads * dv] and the caches must share a dtype")
+    if n_head % G or dv > 256 or dk > 512:
+        raise KernelError(f"attention_scored: {n_head} heads over {G}, keys of {dk}, values of {dv} are not taken")
+    if block_tables.dim() != 2 or block_tables.shape[0] < ctx.n_seqs:
+        raise KernelError("attention_scored: block_tables must be [requests, max_blocks]")
+    _i32(block_tables, "block_tables")
+    _i32(ctx.tok_seq, "tok_seq", n)
+    _i32(ctx.positions, "positions", n)
+    max_dist = 0
+    if bias_table is not None:
+        _dev(bias_table, "bias_table")
+        if bias_table.dtype != torch.float32 or bias_table.dim() != 2 or bias_table.shape[1] != n_head or not bias_table.is_contiguous():
+            raise KernelError(f"attention_scored: the bias table must be contiguous float32 [distances, {n_head}]")
+        max_dist = bias_table.shape[0] - 1
+    gs = 0
+    if gate is not None:
+        gs = _rows(gate, "gate")
+        if gate.dtype != torch.float32 or tuple(gate.shape) != (n, n_head * dv):
+            raise KernelError("attention_scored: the gate must be float32 rows [n, heads * dv]")
+    _lib.call("liyab_attention_scored", out.data_ptr(), so, q.data_ptr(), sq, k_cache.data_ptr(), v_cache.data_ptr(), dtype_code(q.dtype),
+              block_tables.data_ptr(), block_tables.shape[1], ctx.tok_seq.data_ptr(), ctx.positions.data_ptr(), n, float(scale), float(softcap),
+              int(window), _ptr(bias_table), max_dist, _ptr(gate), gs, n_head, G, dk, dv, page, _pages(k_cache, num_pages), _stream())

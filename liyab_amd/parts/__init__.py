@@ -15,4 +15,4 @@ from .registry import (  # noqa: F401
     register_position,
 )
 from .norms import Normed, as_tensor  # noqa: F401
-from . import attention, block, conv, embeddings, feedforward, head, latent_attention, norms, routed  # noqa: F401  (register themselves)
+from . import attention, block, conv, embeddings, feedforward, head, latent_attention, norms, recurrent, routed, scored_attention, side_by_side  # noqa: F401  (register themselves)

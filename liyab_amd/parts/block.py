@@ -72,6 +72,37 @@ class PreNormBlock:
 register_block("pre_norm", PreNormBlock)
 
 
+class ParallelBlock:
+    """h = norm(x); x += mixer(h) + ffn(h): one norm, and both sublayers read its output. Each sublayer adds its result into
+    the 32-bit stream from its last product's epilogue; h is a buffer of its own, so the second sublayer still reads the
+    norm of the stream as the layer found it."""
+
+    replayable = True
+    takes_padding_rows = True
+    takes_pending = False
+
+    def __init__(self, spec, mixer, ffn, norm_mixer, norm_ffn):
+        if norm_ffn is not None:
+            raise ValueError("a parallel block has one norm (norm_mixer)")
+        self.mixer, self.ffn, self.norm_mixer, self.norm_ffn = mixer, ffn, norm_mixer, None
+        self.mixer_phase = getattr(getattr(spec, "mixer", None), "kind", "mixer")
+        self.ffn_phase = getattr(getattr(spec, "ffn", None), "kind", "ffn")
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, cache, state, writes_cache: bool = True):
+        if ctx.phases is not None:
+            ctx.phases.mark(self.mixer_phase)
+        h = self.norm_mixer.forward(x, ctx, name="block_in")
+        self.mixer.forward(h, ctx, cache, state, x, writes_cache=writes_cache)
+        if self.ffn is not None:
+            if ctx.phases is not None:
+                ctx.phases.mark(self.ffn_phase)
+            self.ffn.forward(h, ctx, x)
+        return None
+
+
+register_block("parallel", ParallelBlock)
+
+
 class PostNormGatedBlock:
     """x += norm_mixer(g1 * mixer(conv(x))); x += norm_ffn(g2 * ffn(x)): the sublayers read the stream
     itself, and the norms stand on their results. g = sigmoid(W x + b) from the stream as the sublayer

@@ -2,6 +2,8 @@
 
 from __future__ import annotations
 
+from typing import Optional
+
 import torch
 
 from .base import StepContext, settled
@@ -49,3 +51,42 @@ class DenseFFN:
 
 
 register_ffn("dense_ffn", DenseFFN)
+
+
+class ClampedGLU:
+    """down(g * sigmoid(slope * g) * (u + shift)) with g = min(Wg h, limit) and u = clamp(Wu h, -limit, limit): the two
+    projections run as one product [gate | up] whose 32-bit sums the activation kernel reads, so that the clamps and the
+    gate see unrounded values; the inner rows are rounded once, for the second product."""
+
+    replayable = True
+    takes_padding_rows = True
+
+    def __init__(self, spec, store, dtype: torch.dtype):
+        self.dtype = dtype
+        self.width, self.inner = spec.width, spec.inner
+        self.limit, self.slope, self.shift = float(spec.limit), float(spec.slope), float(spec.shift)
+        if not self.limit > 0:
+            raise ValueError(f"clamped feed-forward: a limit of {self.limit}")
+        t = spec.tensors
+        self.in_weight = store.fetch_joined([t["gate"], t["up"]], [(self.inner, self.width)] * 2, "matrix", "rows")
+        self.down_weight = store.fetch(t["down"], (self.width, self.inner), "matrix")
+
+    def forward(self, h, ctx: StepContext, residual: Optional[torch.Tensor], out: Optional[torch.Tensor] = None):
+        """Adds the result into `residual` (float32 [n, width]), or leaves it in `out`."""
+        from ..kernels import ops
+        from .norms import as_tensor
+
+        h = as_tensor(h)
+        n = h.shape[0]
+        gu = ctx.workspace.get("glu_in", (n, 2 * self.inner), torch.float32)
+        linear(h, self.in_weight, None, out=gu)
+        inner = ctx.workspace.get("ffn_inner", (n, self.inner), self.dtype)
+        ops.glu_clamped(inner, gu, self.limit, self.slope, self.shift)
+        if out is not None:
+            linear(inner, self.down_weight, None, out=out)
+        else:
+            linear(inner, self.down_weight, None, residual=settled(residual))
+        return None
+
+
+register_ffn("clamped_glu", ClampedGLU)

@@ -110,3 +110,29 @@ class RMSNorm:
 
 
 register_norm("rmsnorm", RMSNorm)
+
+
+class DynamicTanh:
+    """y = tanh(alpha * x) * weight + bias: a norm that takes no mean and no variance, with one learned scalar alpha (kept
+    on the device; the kernel reads it there). `rows` gathers (the final norm runs on the wanted rows only)."""
+
+    replayable = True
+    takes_padding_rows = True
+
+    def __init__(self, spec, store, dtype: torch.dtype):
+        self.width = spec.width
+        self.dtype = dtype
+        t = spec.tensors
+        self.weight = store.fetch(t["weight"], (self.width,), "vector") if "weight" in t else None
+        self.bias = store.fetch(t["bias"], (self.width,), "vector") if "bias" in t else None
+        self.alpha = store.fetch(t["alpha"], (), "vector").reshape(1)
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, rows: Optional[torch.Tensor] = None,
+                n_rows: Optional[int] = None, name: str = "normed") -> torch.Tensor:
+        n = x.shape[-2] if rows is None else (n_rows if n_rows is not None else rows.numel())
+        out = ctx.workspace.get(name, (n, self.width), self.dtype)
+        ops.dyt(out, x, self.weight, self.bias, self.alpha, rows=rows)
+        return out
+
+
+register_norm("dyt", DynamicTanh)

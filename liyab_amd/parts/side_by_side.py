@@ -1,0 +1,70 @@
+"""Two mixers that read the same input, their results joined."""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..kernels import ops
+from .base import StepContext, settled
+from .norms import as_tensor
+from .registry import build_part, register_mixer
+
+
+class SideBySide:
+    """result = weight * (left(h) / rms(left(h)) * w_left + right(h) / rms(right(h)) * w_right), the root mean squares over
+    the model's width. The two mixers are parts of the mixer registry that can leave their result to the caller
+    (`forward(..., out=)`); at most one of them keeps rows in the pages and at most one keeps state, and this part passes
+    the layer's cache and slot on to the one that does."""
+
+    replayable = True
+
+    @property
+    def takes_padding_rows(self) -> bool:
+        return bool(getattr(self.left, "takes_padding_rows", False)) and bool(getattr(self.right, "takes_padding_rows", False))
+
+    def __init__(self, spec, store, dtype: torch.dtype):
+        self.dtype = dtype
+        self.width, self.eps, self.weight = spec.width, float(spec.eps), float(spec.weight)
+        self.left = build_part("mixer", spec.left, store, dtype)
+        self.right = build_part("mixer", spec.right, store, dtype)
+        for part in (self.left, self.right):
+            if "out" not in part.forward.__code__.co_varnames:
+                raise ValueError("mixers side by side must be able to leave their result to the caller (forward(..., out=))")
+        if self.left.cache_spec() is not None and self.right.cache_spec() is not None:
+            raise ValueError("mixers side by side: only one of them may keep rows in the pages")
+        if self.left.state_spec() is not None and self.right.state_spec() is not None:
+            raise ValueError("mixers side by side: only one of them may keep state")
+        t = spec.tensors
+        self.left_out = store.fetch(t["left_out"], (self.width,), "vector")
+        self.right_out = store.fetch(t["right_out"], (self.width,), "vector")
+        planners = [p for p in (getattr(self.left, "step_planner", None), getattr(self.right, "step_planner", None)) if p is not None]
+        if len(planners) > 1:
+            raise ValueError("mixers side by side: only one of them may plan a step")
+        if planners:
+            self.step_planner = planners[0]
+
+    def cache_spec(self):
+        return self.left.cache_spec() or self.right.cache_spec()
+
+    def state_spec(self):
+        return self.left.state_spec() or self.right.state_spec()
+
+    def forward(self, h, ctx: StepContext, cache, state, residual: Optional[torch.Tensor], writes_cache: bool = True,
+                out: Optional[torch.Tensor] = None):
+        h = as_tensor(h)
+        n, ws = h.shape[0], ctx.workspace
+        a = ws.get("side_left", (n, self.width), torch.float32)
+        b = ws.get("side_right", (n, self.width), torch.float32)
+        self.left.forward(h, ctx, cache, state, None, writes_cache=writes_cache, out=a)
+        self.right.forward(h, ctx, cache, state, None, writes_cache=writes_cache, out=b)
+        if out is not None:
+            ops.fill_(out, 0)
+            ops.mean_norm_add(out, a, b, self.left_out, self.right_out, self.eps, self.weight)
+        else:
+            ops.mean_norm_add(settled(residual), a, b, self.left_out, self.right_out, self.eps, self.weight)
+        return None
+
+
+register_mixer("side_by_side", SideBySide)

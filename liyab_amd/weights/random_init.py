@@ -46,7 +46,7 @@ def draw(seed: int, name: str, shape: Sequence[int], init: Init) -> torch.Tensor
     """float32 N(init.mean, init.std) of `shape` from the generator of (seed, name)."""
     rng = np.random.Generator(np.random.Philox(key=[seed & 0xFFFFFFFFFFFFFFFF, _name_key(name)]))
     a = rng.standard_normal(size=tuple(int(s) for s in shape), dtype=np.float32)
-    return torch.from_numpy(a * np.float32(init.std) + np.float32(init.mean))
+    return torch.from_numpy(np.asarray(a * np.float32(init.std) + np.float32(init.mean), dtype=np.float32))
 
 
 class DrawingStore:
