@@ -6,7 +6,7 @@
     python bench.py --workload medium16|xl64         # the continuous-batching and the batch-64 workloads of the larger sizes
     python bench.py --link-floor                     # what one dependent kernel of a replayed graph costs at least
     python bench.py --product 4096,4096,16384,8,15   # one product in tiles of 128 x 128 and of 256 x 256
-    python bench.py --design bokulix [--design-sizes small,medium,xl] [--layers L] [--phases]   # Bokulix beside GPT-2 at equal sizes
+    python bench.py --design bokulix|mofulix [--design-sizes small,medium,xl] [--layers L] [--phases]   # that design beside GPT-2 at equal sizes
 
 The default run has GPT-2 small's layer sizes (12 layers, width 768, 12 heads
 of 64, feed-forward 3072, vocabulary 50257, 1024 positions) with random
@@ -404,18 +404,104 @@ def bokulix_prefill_flops(cfg, prompt_lens, logit_rows):
     return flops
 
 
+# -- Mofulix beside GPT-2 at equal sizes --------------------------------------------------------------------
+# The Mofulix of each size has GPT-2's width, layers, vocabulary and head count (heads of 64 everywhere), its layers
+# taking turns as gated attention (as many key heads as query heads, so that attention reads what GPT-2's reads), wkv,
+# and attention with a bias by distance beside a state space (heads of 64 with a state of 64, four taps); the gated
+# feed-forward is two thirds as wide as GPT-2's, which makes its three matrices as large as GPT-2's two.
+def mofulix_config(gpt2_cfg):
+    d, H, F, L = gpt2_cfg["n_embd"], gpt2_cfg["n_head"], gpt2_cfg["n_inner"], gpt2_cfg["n_layer"]
+    hd = d // H
+    ff = max(64, F * 2 // 3 // 64 * 64)
+    mlp = {"kind": "dense", "ff": ff, "limit": 7.0}
+    kinds = [
+        {"type": "attention", "mixer": {"heads": H, "kv_heads": H, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "softcap": 30.0,
+                                        "rot": {"dims": hd, "base": 10000.0, "scaling": {"factor": 4.0, "low": 1.0, "high": 4.0, "original": 2048}}}},
+        {"type": "wkv", "mixer": {"heads": H, "dim": hd, "decay_rank": 64}},
+        {"type": "parallel", "mixer": {"left": {"heads": H, "kv_heads": H, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "bias_max": 128, "bias_rows": 32,
+                                                "q_temp": {"coef": 0.1, "every": 256}},
+                                       "right": {"heads": H, "vdim": hd, "state": 64, "groups": 1, "conv": 4, "norm_groups": 1}}},
+    ]
+    layers = [dict(json.loads(json.dumps(kinds[i % 3])), mlp=dict(mlp)) for i in range(L)]
+    return {"architecture": "Mofulix", "vocab": gpt2_cfg["vocab_size"], "width": d, "embedding": {"scale": 1.0}, "norm": {"eps": 1e-5},
+            "max_positions": gpt2_cfg["n_positions"], "layers": layers}
+
+
+def _mofulix_layer_weights(entry, d):
+    """Matrix elements of a layer (what a step reads of it), and of them those of products (2 flops an element a token)."""
+    m, kind = entry["mixer"], entry["type"]
+    n = 3 * entry["mlp"]["ff"] * d if entry.get("mlp") else 0
+    if kind == "attention":
+        H, G, D = m["heads"], m["kv_heads"], m["dim"]
+        n += (H * D + G * D + H * D) * d + d * H * D
+    elif kind == "wkv":
+        HD, R = m["heads"] * m["dim"], m.get("decay_rank", 16)
+        n += 4 * HD * d + R * d + HD * R + d * HD
+    else:
+        a, b = m["left"], m["right"]
+        n += (a["heads"] * a["dim"] + a["kv_heads"] * (a["dim"] + a["vdim"])) * d + d * a["heads"] * a["vdim"]
+        inner = b["heads"] * b["vdim"]
+        n += (2 * inner + 2 * b["groups"] * b["state"] + b["heads"]) * d + d * inner
+    return n
+
+
+def mofulix_step_bytes(cfg, batch):
+    """The bytes a decode step has to read: every matrix once, the head, the cached keys and values of the attention layers,
+    and the 32-bit state of the recurrent ones (read and written) a request."""
+    def step_bytes(contexts, steps, elt):
+        d, V = cfg["width"], cfg["vocab"]
+        total = V * d * elt
+        seen = sum(sum(c + s + 1 for s in range(steps)) for c in contexts) / max(steps, 1)
+        for entry in cfg["layers"]:
+            m = entry["mixer"]
+            total += _mofulix_layer_weights(entry, d) * elt
+            if entry["type"] == "attention":
+                total += seen * 2 * m["kv_heads"] * m["dim"] * elt
+            elif entry["type"] == "wkv":
+                total += len(contexts) * 2 * m["heads"] * m["dim"] * m["dim"] * 4
+            else:
+                a, b = m["left"], m["right"]
+                total += seen * a["kv_heads"] * (a["dim"] + a["vdim"]) * elt + len(contexts) * 2 * b["heads"] * b["vdim"] * b["state"] * 4
+        return total
+    return step_bytes
+
+
+def mofulix_prefill_flops(cfg, prompt_lens, logit_rows):
+    d, V, n = cfg["width"], cfg["vocab"], sum(prompt_lens)
+    flops = 2.0 * logit_rows * d * V
+    pairs = sum(t * (t + 1) / 2 for t in prompt_lens)
+    for entry in cfg["layers"]:
+        m = entry["mixer"]
+        flops += 2.0 * n * _mofulix_layer_weights(entry, d)
+        if entry["type"] == "attention":
+            flops += 2.0 * pairs * m["heads"] * 2 * m["dim"]
+        elif entry["type"] == "wkv":
+            flops += n * m["heads"] * 6.0 * m["dim"] * m["dim"]  # a token: the state's update and its read, a head
+        else:
+            a, b = m["left"], m["right"]
+            flops += 2.0 * pairs * a["heads"] * (a["dim"] + a["vdim"]) + n * b["heads"] * 6.0 * b["vdim"] * b["state"]
+    return flops
+
+
+DESIGNS = {"bokulix": (lambda gpt2, size: bokulix_config(gpt2, BOKULIX_SHAPES[size]), bokulix_step_bytes, bokulix_prefill_flops),
+           "mofulix": (lambda gpt2, size: mofulix_config(gpt2), mofulix_step_bytes, mofulix_prefill_flops)}
+
+
 def design_run(args):
-    """Bokulix and GPT-2 side by side at each of the named sizes: a prefill of 2,048 tokens (two prompts of 1,024) with its
+    """A design and GPT-2 side by side at each of the named sizes: a prefill of 2,048 tokens (two prompts of 1,024) with its
     share of the matrix peak, and decode steps at batch 1, 8 and 64 with their share of the HBM roofline."""
     from liyab_amd.weights import write_random_model
 
+    make_config, step_bytes_of, flops_of = DESIGNS[args.design]
     short = "bf16" if args.dtype == "bfloat16" else "fp32"
     runs = []
     for size in args.design_sizes.split(","):
         gpt2 = dict(SMALL, **SIZES[size])
         if args.layers:
             gpt2["n_layer"] = args.layers
-        designs = {"gpt2": gpt2, "bokulix": bokulix_config(gpt2, BOKULIX_SHAPES[size])}
+        designs = {"gpt2": gpt2, args.design: make_config(gpt2, size)}
+        if args.design_only:
+            del designs["gpt2"]
         ctx = gpt2["n_positions"]
         k = max(16, min(args.steps, 128, ctx - args.prompt - 16))
         for name, cfg in designs.items():
@@ -424,14 +510,14 @@ def design_run(args):
                 engine = make_engine(d, args.dtype, 64, ctx, page_size=args.page_size, phases=args.phases)
                 lens = [1024, 1024]
                 ptps, pms = prefill_run(engine, cfg, lens)
-                flops = bokulix_prefill_flops(cfg, lens, 2) if name == "bokulix" else prefill_flops(cfg, lens, 2)
+                flops = flops_of(cfg, lens, 2) if name != "gpt2" else prefill_flops(cfg, lens, 2)
                 run = {"design": name, "size": size, "layers": gpt2["n_layer"],
                        "prefill": {"tokens": 2048, "tok_s": round(ptps, 1), "ms": round(pms, 4), "gflop": round(flops / 1e9, 1),
                                    "frac_of_matrix_peak": round(flops / (pms * 1e-3) / MFMA_PEAK[short], 4)}}
                 if args.phases:
                     run["prefill"]["phases_ms"] = {n: round(v / 7, 4) for n, v in engine.phases_ms(reset=True).items()}  # (prefill_run steps 7 times)
                 for b in (1, 8, 64):
-                    bytes_fn = bokulix_step_bytes(cfg, b) if name == "bokulix" else None
+                    bytes_fn = step_bytes_of(cfg, b) if name != "gpt2" else None
                     t, ms, nbytes = decode_run(engine, cfg, b, args.prompt, k, 4, step_bytes=bytes_fn)
                     run[f"decode_b{b}"] = {"tok_s": round(t, 1), "ms_per_step": round(ms, 4), "mbytes_per_step": round(nbytes / 1e6, 1),
                                            "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
@@ -443,7 +529,7 @@ def design_run(args):
                         run[f"decode_b{b}"]["phases_ms"] = {n: round(max(v - prompts.get(n, 0.0), 0.0) / (k + 4), 4) for n, v in whole.items()}
                 runs.append(run)
                 del engine
-    print(json.dumps({"metric": "Bokulix beside GPT-2 at equal layer sizes: prefill of 2,048 tokens and decode steps", "dtype": short,
+    print(json.dumps({"metric": f"{args.design.capitalize()} beside GPT-2 at equal layer sizes: prefill of 2,048 tokens and decode steps", "dtype": short,
                       "data": "synthetic", "page_size": args.page_size, "prompt_len": args.prompt, "runs": runs}))
     return 0
 
@@ -475,8 +561,9 @@ def main():
     ap.add_argument("--link-floor", action="store_true", help="measure what one dependent kernel of a replayed graph costs at least")
     ap.add_argument("--phases", action="store_true", help="device milliseconds per phase of the forward pass (embed, attention, dense_ffn, lm_head) a decode step "
                     "and a prefill of 2,048 tokens, as the reference's command line prints them (tools/liyab_cli.cpp:198-211); steps run kernel by kernel, without graphs")
-    ap.add_argument("--design", default="", choices=["", "bokulix"],
-                    help="bokulix: that design beside GPT-2 at equal layer sizes (prefill and decode, both with their rooflines)")
+    ap.add_argument("--design", default="", choices=["", "bokulix", "mofulix"],
+                    help="bokulix, mofulix: that design beside GPT-2 at equal layer sizes (prefill and decode, both with their rooflines)")
+    ap.add_argument("--design-only", action="store_true", help="with --design: skip the GPT-2 run (for profiling)")
     ap.add_argument("--design-sizes", default="small,medium,xl", help="the sizes --design runs (of small, medium, xl)")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -70,14 +70,18 @@ __device__ __forceinline__ void merge_partial(Partial& a, float mo, float lo, co
     a.m = M;
 }
 
-template <typename T, int LPK, int AD_WAVES, int AD_U>
+// SCORED: the score scale * q . k is worked on before the softmax: a soft cap, cap * tanh(score / cap) (softcap > 0), then
+// a bias by distance, bias_table[min(position - key, max_dist), head] (bias_table given). Without SCORED the three
+// arguments are not read, and the kernel is the one it was.
+template <typename T, int LPK, int AD_WAVES, int AD_U, bool SCORED = false>
 __global__ void __launch_bounds__(64 * AD_WAVES)
 attention_decode_kernel(T* __restrict__ out, int64_t out_stride, const T* __restrict__ q, int64_t q_stride,
                         const T* __restrict__ kc, const T* __restrict__ vc,
                         const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ tok_list,
                         const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, float scale, int window,
                         int n_head, int n_kv_head, int hd, int page_size, int page_shift, int rows_are_requests,
-                        int n_splits, int chunk, float* __restrict__ partials, int num_pages) {
+                        int n_splits, int chunk, float* __restrict__ partials, int num_pages, float softcap = 0.0f,
+                        const float* __restrict__ bias_table = nullptr, int max_dist = 0) {
     constexpr int KPP = 64 / LPK;  // keys per wave and pass
     __shared__ float lds2[2][AD_WAVES][LPK][10];  // the waves' sums, for the first wave to merge; two of them in turn, so that one barrier a split is enough
     const int t = tok_list != nullptr ? tok_list[blockIdx.x] : blockIdx.x;
@@ -155,6 +159,13 @@ attention_decode_kernel(T* __restrict__ out, int64_t out_stride, const T* __rest
             for (int e = 0; e < 8; ++e) d = fmaf(kf[e], qf[e], d);
             d = group_sum<LPK>(d);  // over the lanes that share the key
             s[u] = valid[u] ? d * scale : -INFINITY;
+            if constexpr (SCORED) {
+                if (valid[u]) {
+                    if (softcap > 0.0f) s[u] = softcap * tanhf(s[u] / softcap);
+                    if (bias_table != nullptr)
+                        s[u] += bias_table[static_cast<int64_t>(min(pos - (j0 + u * AD_WAVES * KPP + kg), max_dist)) * n_head + h];
+                }
+            }
             m_new = fmaxf(m_new, s[u]);
         }
         if (m_new == -INFINITY) continue;  // this lane group had no key in this trip (and none before)
@@ -286,12 +297,13 @@ __global__ void attention_merge_kernel(T* __restrict__ out, int64_t out_stride, 
     out[static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * hd + e] = from_float<T>(o / sum);
 }
 
-template <typename T>
+template <typename T, bool SCORED = false>
 int launch_attention_decode(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc, const void* vc,
                             const int* block_tables, int max_blocks, const int* tok_list, const int* tok_seq,
                             const int* tok_pos, int n, float scale, int window, int n_head, int n_kv_head, int hd,
                             int page_size, int n_splits, int chunk, int waves, int rows_are_requests, float* partials,
-                            int leave_splits, int num_pages, hipStream_t stream) {
+                            int leave_splits, int num_pages, hipStream_t stream, float softcap = 0.0f, const float* bias_table = nullptr,
+                            int max_dist = 0) {
     int page_shift = -1;
     for (int b = 0; b < 31; ++b)
         if ((1 << b) == page_size) page_shift = b;
@@ -303,17 +315,17 @@ int launch_attention_decode(void* out, int64_t out_stride, const void* q, int64_
 #define LIYAB_GO(L)                                                                                                  \
     do {                                                                                                             \
         if (waves == 4)                                                                                              \
-            attention_decode_kernel<T, L, 4, 4><<<grid, 256, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
+            attention_decode_kernel<T, L, 4, 4, SCORED><<<grid, 256, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
                                                                     max_blocks, tok_list, tok_seq, tok_pos, scale,   \
-                                                                    window, n_head, n_kv_head, hd, page_size, page_shift, rows_are_requests, n_splits, chunk, partials, num_pages); \
+                                                                    window, n_head, n_kv_head, hd, page_size, page_shift, rows_are_requests, n_splits, chunk, partials, num_pages, softcap, bias_table, max_dist); \
         else if (waves == 8)                                                                                         \
-            attention_decode_kernel<T, L, 8, 4><<<grid, 512, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
+            attention_decode_kernel<T, L, 8, 4, SCORED><<<grid, 512, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
                                                                     max_blocks, tok_list, tok_seq, tok_pos, scale,   \
-                                                                    window, n_head, n_kv_head, hd, page_size, page_shift, rows_are_requests, n_splits, chunk, partials, num_pages); \
+                                                                    window, n_head, n_kv_head, hd, page_size, page_shift, rows_are_requests, n_splits, chunk, partials, num_pages, softcap, bias_table, max_dist); \
         else                                                                                                         \
-            attention_decode_kernel<T, L, 16, sizeof(T) == 2 ? 8 : 4><<<grid, 1024, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
+            attention_decode_kernel<T, L, 16, sizeof(T) == 2 ? 8 : 4, SCORED><<<grid, 1024, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
                                                                       max_blocks, tok_list, tok_seq, tok_pos, scale, \
-                                                                      window, n_head, n_kv_head, hd, page_size, page_shift, rows_are_requests, n_splits, chunk, partials, num_pages); \
+                                                                      window, n_head, n_kv_head, hd, page_size, page_shift, rows_are_requests, n_splits, chunk, partials, num_pages, softcap, bias_table, max_dist); \
     } while (0)
     if (hd <= 8) LIYAB_GO(1);
     else if (hd <= 16) LIYAB_GO(2);
@@ -342,11 +354,11 @@ using namespace liyab;
 // split an equal share of the token's keys; > 0 = split z takes keys [z * chunk, (z + 1) * chunk)
 // of the token's (n_splits * chunk must cover the longest context: keys beyond are not read).
 // num_pages: the pages the caches hold; page ids of the block tables are brought into [0, num_pages).
-extern "C" int liyab_attention_decode(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc,
-                                      const void* vc, int dtype, const int* block_tables, int max_blocks, const int* tok_list,
-                                      const int* tok_seq, const int* tok_pos, int n, float scale, int window,
-                                      int n_head, int n_kv_head, int hd, int page_size, int n_splits, int chunk, int waves,
-                                      int rows_are_requests, float* partials, int leave_splits, int num_pages, hipStream_t stream) {
+static int check_attention_decode(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc, const void* vc, int dtype,
+                                  const int* block_tables, int max_blocks, const int* tok_list, const int* tok_seq, const int* tok_pos, int n,
+                                  int window, int n_head, int n_kv_head, int hd, int page_size, int n_splits, int chunk, int waves,
+                                  int rows_are_requests, float* partials, int leave_splits, int num_pages) {
+
     LIYAB_REQUIRE(num_pages > 0, "attention_decode: the caches hold %d pages", num_pages);
     LIYAB_REQUIRE((out || leave_splits) && q && kc && vc && block_tables && tok_seq && tok_pos, "attention_decode: null pointer");
     LIYAB_REQUIRE(dtype == kBF16 || dtype == kF32, "attention_decode: unknown dtype %d", dtype);
@@ -370,6 +382,17 @@ extern "C" int liyab_attention_decode(void* out, int64_t out_stride, const void*
     LIYAB_REQUIRE(max_blocks <= AD_MAX_BLOCKS, "attention_decode: block tables of %d pages; at most %d are taken", max_blocks, AD_MAX_BLOCKS);
     LIYAB_REQUIRE(!rows_are_requests || tok_list == nullptr, "attention_decode: rows_are_requests does not go with a row list");
     LIYAB_REQUIRE(waves == 4 || waves == 8 || waves == 16, "attention_decode: %d waves per workgroup is not 4, 8 or 16", waves);
+    return 0;
+}
+
+extern "C" int liyab_attention_decode(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc,
+                                      const void* vc, int dtype, const int* block_tables, int max_blocks, const int* tok_list,
+                                      const int* tok_seq, const int* tok_pos, int n, float scale, int window,
+                                      int n_head, int n_kv_head, int hd, int page_size, int n_splits, int chunk, int waves,
+                                      int rows_are_requests, float* partials, int leave_splits, int num_pages, hipStream_t stream) {
+    if (int rc = check_attention_decode(out, out_stride, q, q_stride, kc, vc, dtype, block_tables, max_blocks, tok_list, tok_seq, tok_pos, n, window,
+                                        n_head, n_kv_head, hd, page_size, n_splits, chunk, waves, rows_are_requests, partials, leave_splits, num_pages))
+        return rc;
     if (n == 0) return 0;
     if (dtype == kF32)
         return launch_attention_decode<float>(out, out_stride, q, q_stride, kc, vc, block_tables, max_blocks, tok_list, tok_seq,
@@ -378,6 +401,28 @@ extern "C" int liyab_attention_decode(void* out, int64_t out_stride, const void*
     return launch_attention_decode<bf16_t>(out, out_stride, q, q_stride, kc, vc, block_tables, max_blocks, tok_list, tok_seq,
                                            tok_pos, n, scale, window, n_head, n_kv_head, hd, page_size, n_splits, chunk, waves,
                                            rows_are_requests, partials, leave_splits, num_pages, stream);
+}
+
+// The same with the scores worked on before the softmax: softcap > 0 caps them, cap * tanh(score / cap); bias_table (float
+// [max_dist + 1, n_head]) adds table[min(position - key, max_dist), head].
+extern "C" int liyab_attention_decode_scored(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc,
+                                             const void* vc, int dtype, const int* block_tables, int max_blocks, const int* tok_list,
+                                             const int* tok_seq, const int* tok_pos, int n, float scale, int window,
+                                             int n_head, int n_kv_head, int hd, int page_size, int n_splits, int chunk, int waves,
+                                             int rows_are_requests, float* partials, int leave_splits, int num_pages, float softcap,
+                                             const float* bias_table, int max_dist, hipStream_t stream) {
+    if (int rc = check_attention_decode(out, out_stride, q, q_stride, kc, vc, dtype, block_tables, max_blocks, tok_list, tok_seq, tok_pos, n, window,
+                                        n_head, n_kv_head, hd, page_size, n_splits, chunk, waves, rows_are_requests, partials, leave_splits, num_pages))
+        return rc;
+    LIYAB_REQUIRE(softcap >= 0.0f && (bias_table == nullptr || max_dist >= 0), "attention_decode_scored: a negative cap or distance");
+    if (n == 0) return 0;
+    if (dtype == kF32)
+        return launch_attention_decode<float, true>(out, out_stride, q, q_stride, kc, vc, block_tables, max_blocks, tok_list, tok_seq,
+                                                    tok_pos, n, scale, window, n_head, n_kv_head, hd, page_size, n_splits, chunk, waves,
+                                                    rows_are_requests, partials, leave_splits, num_pages, stream, softcap, bias_table, max_dist);
+    return launch_attention_decode<bf16_t, true>(out, out_stride, q, q_stride, kc, vc, block_tables, max_blocks, tok_list, tok_seq,
+                                                 tok_pos, n, scale, window, n_head, n_kv_head, hd, page_size, n_splits, chunk, waves,
+                                                 rows_are_requests, partials, leave_splits, num_pages, stream, softcap, bias_table, max_dist);
 }
 
 // out[m, h * hd + e] = the splits of (m, h) merged in split order: for splits that

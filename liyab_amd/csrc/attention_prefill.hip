@@ -59,12 +59,16 @@ constexpr int AP_QUERIES = 128; // queries per tile (4 waves x 32)
 constexpr int kDepth = 6;       // blocks of keys and values in flight in registers
 constexpr int AP_MAX_BLOCKS = 2048;  // page ids of a tile's keys are kept in LDS
 
-template <int DB, int QG, int KS, int NS = 1>  // head dimension padded to 32 * DB; 32 * QG queries a tile; KS x NS blocks of keys a step, NS a wave
+// SCORED: the scores are worked on before the softmax: scale * q . k, capped as cap * tanh(. / cap) when softcap > 0, plus
+// bias_table[min(query position - key position, max_dist), head] when a table is given; the exponentials then take the
+// scores as they are. Without SCORED the three arguments are not read, and the kernel is the one it was.
+template <int DB, int QG, int KS, int NS = 1, bool SCORED = false>  // head dimension padded to 32 * DB; 32 * QG queries a tile; KS x NS blocks of keys a step, NS a wave
 __global__ void __launch_bounds__(64 * QG * KS)
 attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
                          const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
                          const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ work, float scale,
-                         int window, int n_head, int n_kv_head, int hd, int page_size, int page_shift, int num_pages) {
+                         int window, int n_head, int n_kv_head, int hd, int page_size, int page_shift, int num_pages,
+                         float softcap = 0.0f, const float* __restrict__ bias_table = nullptr, int max_dist = 0) {
     constexpr int HDP = 32 * DB;
     constexpr int LDK = HDP + 8;  // padded row: 16-byte reads of 16 lanes fall in distinct banks
     constexpr int WAVES = QG * KS, THREADS = 64 * WAVES;
@@ -102,7 +106,7 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
     const int wave_last = pos0 + min(32 * qg + 31, nq - 1);  // the wave's latest query position
     const bool wave_has = 32 * qg < nq;
     const int n_slabs = hd / 16;
-    const float scale2 = scale * 1.4426950408889634f;  // log2(e): exp(x) = 2^(x log2 e)
+    const float scale2 = (SCORED ? 1.0f : scale) * 1.4426950408889634f;  // log2(e): exp(x) = 2^(x log2 e)
 
     QFrag qf[2 * DB];
     {
@@ -212,6 +216,27 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
             // wave sees whole needs no mask. The maximum is taken over the raw scores (the scale is
             // positive); exponentials are 2^(score * scale2 - reference), one fused multiply-add and
             // one v_exp_f32 a score.
+            if constexpr (SCORED) {
+                const float inv_cap = softcap > 0.0f ? 1.0f / softcap : 0.0f;
+#pragma unroll
+                for (int z = 0; z < NS; ++z) {
+                    const int kb = kb0w + z * AP_KEYS;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        float sc = st[z][r] * scale;
+                        if (softcap > 0.0f) {
+                            // tanh(x) = 1 - 2 / (1 + e^(2x)), one hardware exponential and one reciprocal
+                            const float e2 = __builtin_amdgcn_exp2f(2.0f * 1.4426950408889634f * sc * inv_cap);
+                            sc = softcap * (1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + e2));
+                        }
+                        if (bias_table != nullptr) {
+                            const int kp = kb + 8 * (r / 4) + 4 * g2 + r % 4;
+                            sc += bias_table[static_cast<int64_t>(min(max(qpos - kp, 0), max_dist)) * n_head + h];
+                        }
+                        st[z][r] = sc;
+                    }
+                }
+            }
             float bm[NS];
 #pragma unroll
             for (int z = 0; z < NS; ++z) {
@@ -374,10 +399,11 @@ using namespace liyab;
 // work: n_tiles x (request index, first row, first position, queries <= tile), int32; tile = 64 or 128
 // queries (2 or 4 groups of 32); ksplit = 1, 2 or 4 waves share a query group's keys (128-query tiles: 1 or 2).
 // num_pages: the pages the caches hold; page ids of the block tables are brought into [0, num_pages).
-extern "C" int liyab_attention_prefill(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc,
-                                       const void* vc, const int* block_tables, int max_blocks, const int* work,
-                                       int n_tiles, int tile, int ksplit, float scale, int window, int n_head, int n_kv_head, int hd,
-                                       int page_size, int num_pages, hipStream_t stream) {
+template <bool SCORED>
+static int run_attention_prefill(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc,
+                                 const void* vc, const int* block_tables, int max_blocks, const int* work,
+                                 int n_tiles, int tile, int ksplit, float scale, int window, int n_head, int n_kv_head, int hd,
+                                 int page_size, int num_pages, float softcap, const float* bias_table, int max_dist, hipStream_t stream) {
     LIYAB_REQUIRE(out && q && kc && vc && block_tables && work, "attention_prefill: null pointer");
     LIYAB_REQUIRE(num_pages > 0, "attention_prefill: the caches hold %d pages", num_pages);
     LIYAB_REQUIRE(n_tiles >= 0 && n_head > 0 && n_kv_head > 0 && page_size > 0 && max_blocks > 0, "attention_prefill: bad sizes");
@@ -405,8 +431,8 @@ extern "C" int liyab_attention_prefill(void* out, int64_t out_stride, const void
     auto* pk = static_cast<const bf16_t*>(kc);
     auto* pv = static_cast<const bf16_t*>(vc);
 #define LIYAB_RUN(D, Q, S)                                                                                          \
-    attention_prefill_kernel<D, Q, S, (D <= 2 && Q == 4 && S <= 2) ? 2 : 1><<<grid, 64 * Q * S, 0, stream>>>(                          \
-        o, out_stride, pq, q_stride, pk, pv, block_tables, max_blocks, work, scale, window, n_head, n_kv_head, hd, page_size, page_shift, num_pages)
+    attention_prefill_kernel<D, Q, S, (D <= 2 && Q == 4 && S <= 2) ? 2 : 1, SCORED><<<grid, 64 * Q * S, 0, stream>>>(                          \
+        o, out_stride, pq, q_stride, pk, pv, block_tables, max_blocks, work, scale, window, n_head, n_kv_head, hd, page_size, page_shift, num_pages, softcap, bias_table, max_dist)
 #define LIYAB_RUN4(D) LIYAB_RUN(D, 2, 4)
 #define LIYAB_SKIP4(D) (void)0  // four stages of 128 keys do not fit LDS at these head sizes (refused above)
 #define LIYAB_GO(D, FOUR)                           \
@@ -429,4 +455,24 @@ extern "C" int liyab_attention_prefill(void* out, int64_t out_stride, const void
 #undef LIYAB_SKIP4
 #undef LIYAB_RUN
     return check_launch("attention_prefill");
+}
+
+extern "C" int liyab_attention_prefill(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc,
+                                       const void* vc, const int* block_tables, int max_blocks, const int* work,
+                                       int n_tiles, int tile, int ksplit, float scale, int window, int n_head, int n_kv_head, int hd,
+                                       int page_size, int num_pages, hipStream_t stream) {
+    return run_attention_prefill<false>(out, out_stride, q, q_stride, kc, vc, block_tables, max_blocks, work, n_tiles, tile, ksplit, scale, window,
+                                        n_head, n_kv_head, hd, page_size, num_pages, 0.0f, nullptr, 0, stream);
+}
+
+// The same with the scores worked on before the softmax: softcap > 0 caps them, cap * tanh(score / cap); bias_table (float
+// [max_dist + 1, n_head]) adds table[min(query position - key position, max_dist), head].
+extern "C" int liyab_attention_prefill_scored(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc,
+                                              const void* vc, const int* block_tables, int max_blocks, const int* work,
+                                              int n_tiles, int tile, int ksplit, float scale, int window, int n_head, int n_kv_head, int hd,
+                                              int page_size, int num_pages, float softcap, const float* bias_table, int max_dist,
+                                              hipStream_t stream) {
+    LIYAB_REQUIRE(softcap >= 0.0f && (bias_table == nullptr || max_dist >= 0), "attention_prefill_scored: a negative cap or distance");
+    return run_attention_prefill<true>(out, out_stride, q, q_stride, kc, vc, block_tables, max_blocks, work, n_tiles, tile, ksplit, scale, window,
+                                       n_head, n_kv_head, hd, page_size, num_pages, softcap, bias_table, max_dist, stream);
 }

@@ -79,6 +79,16 @@ int liyab_moe_route_align(const float* logits, int64_t ld, int n, int n_experts,
 int liyab_moe_align(const int* ids, int n_entries, int n_experts, int block, int* rows_list, int* tile_group, int max_tiles,
                     hipStream_t stream);
 
+int liyab_attention_decode_scored(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc, const void* vc, int dtype,
+                                  const int* block_tables, int max_blocks, const int* tok_list, const int* tok_seq, const int* tok_pos, int n,
+                                  float scale, int window, int n_head, int n_kv_head, int hd, int page_size, int n_splits, int chunk,
+                                  int waves, int rows_are_requests, float* partials, int leave_splits, int num_pages, float softcap,
+                                  const float* bias_table, int max_dist, hipStream_t stream);
+int liyab_attention_prefill_scored(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc, const void* vc,
+                                   const int* block_tables, int max_blocks, const int* work, int n_tiles, int tile, int ksplit, float scale,
+                                   int window, int n_head, int n_kv_head, int hd, int page_size, int num_pages, float softcap,
+                                   const float* bias_table, int max_dist, hipStream_t stream);
+int liyab_gate_rows(void* x, int dtype, int64_t ldx, const float* gate, int64_t ldg, int n, int d, hipStream_t stream);
 int liyab_dyt(void* out, int out_dtype, const float* x, const float* w, const float* b, const float* alpha, const int* rows, int n, int d,
               hipStream_t stream);
 int liyab_glu_clamped(void* out, int out_dtype, const float* gu, int64_t ld, int n, int ff, float limit, float slope, float shift,

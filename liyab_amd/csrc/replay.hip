@@ -96,6 +96,9 @@ static const Entry kEntries[] = {
     LIYAB_ENTRY(liyab_moe_route),
     LIYAB_ENTRY(liyab_moe_align),
     LIYAB_ENTRY(liyab_moe_route_align),
+    LIYAB_ENTRY(liyab_attention_decode_scored),
+    LIYAB_ENTRY(liyab_attention_prefill_scored),
+    LIYAB_ENTRY(liyab_gate_rows),
     LIYAB_ENTRY(liyab_dyt),
     LIYAB_ENTRY(liyab_glu_clamped),
     LIYAB_ENTRY(liyab_activate),

@@ -82,6 +82,11 @@ _SIGNATURES = {
     "liyab_moe_route": [P, c_int64, c_int, c_int, c_int, P, P, P],
     "liyab_moe_align": [P, c_int, c_int, c_int, P, P, c_int, P],
     "liyab_moe_route_align": [P, c_int64, c_int, c_int, c_int, P, P, c_int, P, P, c_int, P],
+    "liyab_attention_decode_scored": [P, c_int64, P, c_int64, P, P, c_int, P, c_int, P, P, P, c_int, c_float, c_int, c_int, c_int,
+                                      c_int, c_int, c_int, c_int, c_int, c_int, P, c_int, c_int, c_float, P, c_int, P],
+    "liyab_attention_prefill_scored": [P, c_int64, P, c_int64, P, P, P, c_int, P, c_int, c_int, c_int, c_float, c_int, c_int,
+                                       c_int, c_int, c_int, c_int, c_float, P, c_int, P],
+    "liyab_gate_rows": [P, c_int, c_int64, P, c_int64, c_int, c_int, P],
     "liyab_dyt": [P, c_int, P, P, P, P, P, c_int, c_int, P],
     "liyab_glu_clamped": [P, c_int, P, c_int64, c_int, c_int, c_float, c_float, c_float, P],
     "liyab_activate": [P, c_int, c_int64, P, c_int64, c_int, c_int, c_int, P],

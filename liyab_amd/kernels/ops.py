@@ -763,7 +763,7 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, 
                      scale: float, window: int = 0, n_splits: int = 1, partials: Optional[torch.Tensor] = None,
                      tok_list: Optional[torch.Tensor] = None, n_tokens: Optional[int] = None, waves: int = 4,
                      rows_are_requests: bool = False, leave_splits: bool = False, chunk: int = 0,
-                     num_pages: Optional[int] = None) -> None:
+                     num_pages: Optional[int] = None, softcap: float = 0.0, bias_table: Optional[torch.Tensor] = None) -> None:
     """Each token on its own over its request's cache (bfloat16, or float32 throughout), its keys cut into `n_splits`.
     With `tok_list` (int32) only those rows are computed. `rows_are_requests`: row t belongs to
     request t (every request brings one token), which saves the kernel a lookup. With
@@ -771,7 +771,8 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, 
     splits, head size + 4], keeps each split's weighted values, maximum and sum for a reader
     that merges them (`gemm_att_parts`). `chunk` > 0: split z takes keys [z * chunk, (z + 1) * chunk) of a
     token's keys instead of an equal share (`n_splits * chunk` must cover the longest context): a token's
-    sums then follow from its position alone."""
+    sums then follow from its position alone. `softcap` > 0: scores become cap * tanh(score / cap); `bias_table` (float32
+    [distances, heads]): + table[min(position - key, distances - 1), head]."""
     if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or not k_cache.is_contiguous() or not v_cache.is_contiguous():
         raise KernelError("attention: caches must be contiguous [pages, kv_heads, page_size, head_dim] of one shape")
     _, hkv, page, hd = k_cache.shape
@@ -797,10 +798,24 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, 
         need = n * n_head * n_splits * (hd + 4)
         if partials is None or partials.dtype != torch.float32 or partials.numel() < need or not partials.is_contiguous():
             raise KernelError(f"attention_decode: {n_splits} splits need {need} float32 of partials")
-    _lib.call("liyab_attention_decode", out.data_ptr(), os_, q.data_ptr(), qs, k_cache.data_ptr(), v_cache.data_ptr(),
-              dtype_code(q.dtype), block_tables.data_ptr(), block_tables.shape[1], _ptr(tok_list), tok_seq.data_ptr(), tok_pos.data_ptr(),
-              n, float(scale), int(window), n_head, hkv, hd, page, n_splits, int(chunk), waves, 1 if rows_are_requests else 0,
-              _ptr(partials), 1 if leave_splits else 0, _pages(k_cache, num_pages), _stream())
+    args = (out.data_ptr(), os_, q.data_ptr(), qs, k_cache.data_ptr(), v_cache.data_ptr(),
+            dtype_code(q.dtype), block_tables.data_ptr(), block_tables.shape[1], _ptr(tok_list), tok_seq.data_ptr(), tok_pos.data_ptr(),
+            n, float(scale), int(window), n_head, hkv, hd, page, n_splits, int(chunk), waves, 1 if rows_are_requests else 0,
+            _ptr(partials), 1 if leave_splits else 0, _pages(k_cache, num_pages))
+    if softcap > 0 or bias_table is not None:
+        _lib.call("liyab_attention_decode_scored", *args, float(softcap), _ptr(bias_table), _bias_rows(bias_table, n_head) - 1, _stream())
+    else:
+        _lib.call("liyab_attention_decode", *args, _stream())
+
+
+def _bias_rows(bias_table: Optional[torch.Tensor], n_head: int) -> int:
+    """The rows of a bias-by-distance table, float32 [distances, heads] on the device (1 for none)."""
+    if bias_table is None:
+        return 1
+    _dev(bias_table, "bias_table")
+    if bias_table.dtype != torch.float32 or bias_table.dim() != 2 or bias_table.shape[1] != n_head or bias_table.shape[0] < 1 or not bias_table.is_contiguous():
+        raise KernelError(f"attention: the bias table must be contiguous float32 [distances, {n_head}], got {tuple(bias_table.shape)} {bias_table.dtype}")
+    return bias_table.shape[0]
 
 
 def attention_merge(out: torch.Tensor, partials: torch.Tensor) -> None:
@@ -818,7 +833,8 @@ def attention_merge(out: torch.Tensor, partials: torch.Tensor) -> None:
 
 def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                       block_tables: torch.Tensor, work: torch.Tensor, n_tiles: int, *, n_head: int, scale: float,
-                      window: int = 0, tile: int = 128, ksplit: int = 1, num_pages: Optional[int] = None) -> None:
+                      window: int = 0, tile: int = 128, ksplit: int = 1, num_pages: Optional[int] = None, softcap: float = 0.0,
+                      bias_table: Optional[torch.Tensor] = None) -> None:
     """Tiles of up to `tile` (64 or 128) consecutive queries of one request over its bfloat16
     cache, on the matrix cores; `ksplit` waves (1, 2, or 4 with tiles of 64) share the keys of
     32 queries. work: int32 [n_tiles, 4] = (request index, first row, first
@@ -837,9 +853,13 @@ def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
     if block_tables.dim() != 2 or block_tables.dtype != torch.int32 or not block_tables.is_contiguous():
         raise KernelError("attention: block_tables must be contiguous int32 [requests, max_blocks]")
     _i32(work, "work", 4 * n_tiles)
-    _lib.call("liyab_attention_prefill", out.data_ptr(), os_, q.data_ptr(), qs, k_cache.data_ptr(), v_cache.data_ptr(),
-              block_tables.data_ptr(), block_tables.shape[1], work.data_ptr(), n_tiles, int(tile), int(ksplit), float(scale), int(window),
-              n_head, hkv, hd, page, _pages(k_cache, num_pages), _stream())
+    args = (out.data_ptr(), os_, q.data_ptr(), qs, k_cache.data_ptr(), v_cache.data_ptr(),
+            block_tables.data_ptr(), block_tables.shape[1], work.data_ptr(), n_tiles, int(tile), int(ksplit), float(scale), int(window),
+            n_head, hkv, hd, page, _pages(k_cache, num_pages))
+    if softcap > 0 or bias_table is not None:  # (see attention_decode)
+        _lib.call("liyab_attention_prefill_scored", *args, float(softcap), _ptr(bias_table), _bias_rows(bias_table, n_head) - 1, _stream())
+    else:
+        _lib.call("liyab_attention_prefill", *args, _stream())
 
 
 PREFILL_KSPLIT4_WORK = 256  # tiles x heads up to which four waves share a tile of 64 queries' keys
@@ -923,15 +943,17 @@ def attention_takes(head_dim: int) -> bool:
 
 def attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
               block_tables: torch.Tensor, ctx, *, n_head: int, scale: float, window: int = 0,
-              splits_ok: bool = False) -> Optional[torch.Tensor]:
+              splits_ok: bool = False, softcap: float = 0.0, bias_table: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
     """Attention of the step's tokens over their requests' cached keys and values; the kernel
     is chosen from the step's shape (`ctx` is the step's StepContext; `ctx.plans["attention"]`
     says how the step's tokens are cut, see parts/attention.py; without it every token goes to
     the plain kernel). With `splits_ok`, a step of few tokens may leave `out` unwritten and
     return the splits of each (token, head) pair instead, float32 [tokens, heads, splits, head
-    size + 4], for `gemm_att_parts`."""
+    size + 4], for `gemm_att_parts`. `softcap`, `bias_table`: what is done to the scores before the softmax (see
+    `attention_decode`); every kernel below does the same."""
     hd = k_cache.shape[3]
     host = ctx.host
+    scored = dict(softcap=softcap, bias_table=bias_table) if softcap > 0 or bias_table is not None else {}
     plan = ctx.plans.get("attention")
     fast = (plan is not None and q.dtype == torch.bfloat16 and hd % 8 == 0 and q.stride(0) % 8 == 0
             and out.stride(0) % 8 == 0)
@@ -944,7 +966,7 @@ def attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache
         attention_decode(out, q, k_cache, v_cache, block_tables, ctx.tok_seq, ctx.positions, n_head=n_head,
                          scale=scale, window=window, n_splits=splits, partials=partials, waves=waves,
                          tok_list=tok_list, n_tokens=n if tok_list is not None else None,
-                         rows_are_requests=tok_list is None and host.max_q_len == 1)
+                         rows_are_requests=tok_list is None and host.max_q_len == 1, **scored)
 
     if (plan is not None and block_tables.shape[1] <= 2048
             and (fast and _invariant or q.dtype == torch.float32 and hd % 8 == 0 and q.stride(0) % 4 == 0 and out.stride(0) % 4 == 0)):
@@ -965,7 +987,7 @@ def attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache
         partials = ctx.workspace.get("attn_partials", (n * n_head * splits * (hd + 4),), torch.float32) if splits > 1 else None
         attention_decode(out, q, k_cache, v_cache, block_tables, ctx.tok_seq, ctx.positions, n_head=n_head, scale=scale,
                          window=window, n_splits=splits, partials=partials, waves=4, chunk=chunk,
-                         rows_are_requests=host.max_q_len == 1)
+                         rows_are_requests=host.max_q_len == 1, **scored)
         return None
     if fast and plan.mode == "decode" and block_tables.shape[1] <= 2048:
         n = out.shape[0]
@@ -974,7 +996,7 @@ def attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache
             partials = ctx.workspace.get("attn_partials", (n, n_head, splits, hd + 4), torch.float32)
             attention_decode(out, q, k_cache, v_cache, block_tables, ctx.tok_seq, ctx.positions, n_head=n_head,
                              scale=scale, window=window, n_splits=splits, partials=partials, waves=waves,
-                             rows_are_requests=host.max_q_len == 1, leave_splits=True)
+                             rows_are_requests=host.max_q_len == 1, leave_splits=True, **scored)
             return partials
         decode(None, n)
         return None
@@ -987,10 +1009,13 @@ def attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache
             # (heads past 96: two waves a query group at every size, 185 against 217 us for 16 x 1,024 tokens of 12 heads of 128)
             ksplit = (4 if plan.tile == 64 and hd <= 64 and work <= PREFILL_KSPLIT4_WORK else 2) if work <= 256 or hd > 96 else 1
             attention_prefill(out, q, k_cache, v_cache, block_tables, plan.work, plan.n_tiles, n_head=n_head,
-                              scale=scale, window=window, tile=plan.tile, ksplit=ksplit)
+                              scale=scale, window=window, tile=plan.tile, ksplit=ksplit, **scored)
         if plan.n_single:
             decode(plan.single_rows, plan.n_single)
         return
+    if scored:
+        attention_scored(out, q, k_cache, v_cache, block_tables, ctx, n_head=n_head, scale=scale, window=window, **scored)
+        return None
     attention_generic(out, q, k_cache, v_cache, block_tables, ctx.tok_seq, ctx.positions, n_head=n_head, scale=scale,
                       window=window)
 
@@ -1520,3 +1545,12 @@ def attention_scored(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, 
     _lib.call("liyab_attention_scored", out.data_ptr(), so, q.data_ptr(), sq, k_cache.data_ptr(), v_cache.data_ptr(), dtype_code(q.dtype),
               block_tables.data_ptr(), block_tables.shape[1], ctx.tok_seq.data_ptr(), ctx.positions.data_ptr(), n, float(scale), float(softcap),
               int(window), _ptr(bias_table), max_dist, _ptr(gate), gs, n_head, G, dk, dv, page, _pages(k_cache, num_pages), _stream())
+
+
+def gate_rows(x: torch.Tensor, gate: torch.Tensor) -> None:
+    """x *= sigmoid(gate) in place; x rows in float32 or bfloat16, gate float32 rows of the same shape (columns of wider
+    rows are fine)."""
+    ldx, ldg = _rows(x, "x"), _rows(gate, "gate")
+    if gate.dtype != torch.float32 or gate.shape != x.shape:
+        raise KernelError("gate_rows: the gate must be float32 and of x's shape")
+    _lib.call("liyab_gate_rows", x.data_ptr(), dtype_code(x.dtype), ldx, gate.data_ptr(), ldg, x.shape[0], x.shape[1], _stream())

@@ -12,6 +12,7 @@ from ..cache.pages import KVSpec
 from ..cache.storage import LayerCache
 from ..errors import Unsupported
 from ..kernels import ops
+from .attention import AttentionStepPlanner
 from .base import StepContext, settled
 from .linear import linear
 from .norms import as_tensor
@@ -61,6 +62,7 @@ class ScoredAttention:
 
     replayable = True
     takes_padding_rows = True  # (slot -1: nothing of theirs is cached, and no other row attends to them)
+    step_planner = AttentionStepPlanner()  # the same cut of a step's tokens as attention's: ctx.plans["attention"]
 
     def __init__(self, spec, store, dtype: torch.dtype):
         self.dtype = dtype
@@ -133,9 +135,18 @@ class ScoredAttention:
                        n_head=H, q_norm=self.q_norm, k_norm=self.k_norm, eps=self.eps, freqs=self.freqs, rot_dims=self.rot_dims,
                        temp_coef=self.temp_coef, temp_every=self.temp_every)
         att = ws.get("scored_att", (n, H * V), self.dtype)
-        ops.attention_scored(att, q, cache.k, cache.v, group.block_tables, ctx, n_head=H, scale=self.scale, softcap=self.softcap,
-                             window=self.window, bias_table=self.bias_table,
-                             gate=proj[:, self.gate_off:self.gate_off + H * V] if self.gated else None)
+        gate = proj[:, self.gate_off:self.gate_off + H * V] if self.gated else None
+        if D == V:
+            # keys and values of one width: the paged attention kernels of the engine (tiles of a prompt's queries on the matrix
+            # cores, single tokens in splits, the 32-bit form), which cap and bias the scores when asked to
+            splits = ops.attention(att, q, cache.k, cache.v, group.block_tables, ctx, n_head=H, scale=self.scale, window=self.window,
+                                   softcap=self.softcap, bias_table=self.bias_table)
+            assert splits is None
+            if gate is not None:
+                ops.gate_rows(att, gate)
+        else:
+            ops.attention_scored(att, q, cache.k, cache.v, group.block_tables, ctx, n_head=H, scale=self.scale, softcap=self.softcap,
+                                 window=self.window, bias_table=self.bias_table, gate=gate)
         if out is not None:
             linear(att, self.out_weight, None, out=out)
         else:

@@ -367,10 +367,11 @@ def test_rotary_frequencies_follow_the_stretch():
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("m", [biased(4, 2, 16, 24, 12, 40, q_temp=(0.3, 7)), biased(3, 3, 6, 10, 9, 50), biased(2, 1, 8, 8, 6, 7, q_temp=(1.0, 3)),
-                               biased(1, 1, 32, 16, 32, 100), biased(2, 2, 64, 32, 4, 3, q_temp=(0.5, 64))])
+                               biased(1, 1, 32, 16, 32, 100), biased(2, 2, 64, 32, 4, 3, q_temp=(0.5, 64)),
+                               biased(4, 1, 16, 16, 10, 30, q_temp=(0.5, 5)), biased(2, 2, 64, 64, 32, 120), biased(3, 1, 8, 8, 7, 11)])
 def test_biased_attention_alone_in_portions(dtype, m):
-    """Keys and values of different widths, the query's factor across several of its steps, the bias by distance over all
-    its rows and past its last."""
+    """Keys and values of different widths and of one width (which the matrix-core kernels take), the query's factor across
+    several of its steps, the bias by distance over all its rows and past its last."""
     entry = layer("parallel", {"left": m, "right": space(1, 8, 4, 1, 2, 1)})
     p = _Layer(dtype, entry, width=72)
     rng = np.random.default_rng(7)
@@ -403,14 +404,14 @@ def test_distance_rows_follow_the_twin():
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("row", [3, 5, 7, 8, 11])
-@pytest.mark.parametrize("page_size", [8, 16])
-def test_a_bias_row_that_stands_out_at_its_edges(dtype, row, page_size):
+@pytest.mark.parametrize("page_size,dk,dv", [(8, 8, 12), (16, 8, 12), (16, 16, 16)])
+def test_a_bias_row_that_stands_out_at_its_edges(dtype, row, page_size, dk, dv):
     """One row of the distance table is far above the others and the scores themselves are small, so that a query's result is
     nearly the mean of the values at that row's distances: a distance counted one off, or a row's edge one off, shows in
     full. Rows below the table's half (one distance each), logarithmic rows, and the last row (every distance from the
     far edge on, hundreds back), in prompts' portions and decoded alone."""
     rows, far, H = 12, 40, 2
-    m = biased(H, 1, 8, 12, rows, far, scale=0.01)
+    m = biased(H, 1, dk, dv, rows, far, scale=0.01)
     rel = torch.zeros(rows, H)
     rel[row, 0] = 14.0
     rel[(row + 3) % rows, 1] = 14.0
