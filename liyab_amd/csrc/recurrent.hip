@@ -67,90 +67,157 @@ struct ScanArgs {
     int G, inner;
 };
 
-template <int MODE, int REG, typename OutT>
+// PF: elements a thread fetches ahead of each staged array (0: none are fetched ahead; the staging loop takes any size).
+// With PF > 0 the next chunk's values are asked for before the current chunk is computed and written to LDS after it, so
+// that a chunk's trip to memory hides behind the chunk before.
+template <int MODE, int REG, int PF, typename OutT>
 __global__ void __launch_bounds__(SCAN_THREADS)
 scan_kernel(ScanArgs a) {
-    extern __shared__ float lds[];
+    extern __shared__ __attribute__((aligned(16))) float lds[];
     const int s = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
     const int R = a.rows, C = a.cols, CL = a.col_lanes;
     const int n_rb = SCAN_THREADS / CL;
-    const int Rp = n_rb * a.rows_per;  // rows as staged: zeros behind the last
+    const int Rp = n_rb * a.rows_per;  // rows as staged: zeros behind the last (rows_per is a multiple of 4)
     float* decay = lds;                           // [CHUNK][Rp]
     float* inr = decay + SCAN_CHUNK * Rp;         // [CHUNK][Rp]
     float* qr = inr + SCAN_CHUNK * Rp;            // [CHUNK][Rp]
     float* val = qr + SCAN_CHUNK * Rp;            // [CHUNK][CL]
     float* part = val + SCAN_CHUNK * CL;          // [CHUNK][n_rb][CL]
-    float* bonus = part + SCAN_CHUNK * SCAN_THREADS;  // [Rp] (wkv)
 
     const int begin = a.seq_starts[s], end = a.seq_starts[s + 1];
     const int slot = a.state_slots[s];
     const bool slot_ok = slot >= 0 && slot < a.n_slots;
-    const int j = tid % CL, rb = tid / CL;
+    const int cl_shift = __builtin_ctz(CL);  // (CL is a power of two)
+    const int j = tid & (CL - 1), rb = tid >> cl_shift;
     const int i0 = rb * a.rows_per;
     float* S_glob = a.state + static_cast<int64_t>(slot_ok ? slot : 0) * a.state_stride + static_cast<int64_t>(h) * R * C;
     const bool fresh = a.positions[begin] == 0;
 
-    float S[REG];
+    float S[REG], bonus[MODE == 0 ? REG : 1];
 #pragma unroll
     for (int ii = 0; ii < REG; ++ii) {
         const int i = i0 + ii;
         S[ii] = (ii < a.rows_per && i < R && j < C && slot_ok && !fresh) ? S_glob[static_cast<int64_t>(i) * C + j] : 0.0f;
-    }
-    if (MODE == 0) {
-        for (int i = tid; i < Rp; i += SCAN_THREADS) bonus[i] = i < R ? a.u[h * R + i] : 0.0f;
+        if (MODE == 0) bonus[ii] = (ii < a.rows_per && i < R) ? a.u[h * R + i] : 0.0f;
     }
     const int g = MODE == 1 ? h / (a.H / a.G) : 0;
     const float neg_A = MODE == 1 ? -expf(a.A_log[h]) : 0.0f;
     const float dskip = MODE == 1 ? a.Dskip[h] : 0.0f;
+    const float dtb = MODE == 1 ? a.dt_bias[h] : 0.0f;
+
+    // What a chunk's staged element (token tt of the chunk, row i / column jj) is made of, as it lies in memory. The loads stand
+    // under no branch (a load under a branch is waited for where the branch ends): a token or a row past the end is fetched
+    // from the last one's address and masked when it is staged.
+    auto raw_rows = [&](int c0, int len, int tt, int i, float& d, float& x, float& q) {
+        const int64_t t = c0 + min(tt, len - 1);
+        const int ic = min(i, R - 1);
+        if (MODE == 0) {
+            const int64_t at = t * a.ld + h * R + ic;
+            d = a.wraw[at] + a.w0[h * R + ic];
+            x = a.k[at];
+            q = a.r[at];
+        } else {
+            d = a.dtraw[t * a.ldp + h];
+            x = a.xbc[t * a.ldx + a.inner + g * R + ic];
+            q = a.xbc[t * a.ldx + a.inner + a.G * R + g * R + ic];
+        }
+    };
+    auto raw_val = [&](int c0, int len, int tt, int jj) {
+        const int64_t t = c0 + min(tt, len - 1);
+        const int jc = min(jj, C - 1);
+        return MODE == 0 ? a.v[t * a.ld + h * C + jc] : a.xbc[t * a.ldx + h * C + jc];
+    };
+    auto raw_gate = [&](int c0, int len, int tt, int jj) {
+        return a.gate[static_cast<int64_t>(c0 + min(tt, len - 1)) * a.ld + h * C + min(jj, C - 1)];
+    };
+    auto put_rows = [&](int len, int tt, int i, float d, float x, float q) {
+        if (tt < len) {
+            const int e = tt * Rp + i;
+            const bool real = i < R;
+            if (MODE == 0) {
+                decay[e] = real ? expf(-expf(d)) : 0.0f;
+                inr[e] = real ? x : 0.0f;
+            } else {
+                const float dt = softplus_f(d + dtb);
+                decay[e] = real ? expf(neg_A * dt) : 0.0f;
+                inr[e] = real ? dt * x : 0.0f;
+            }
+            qr[e] = real ? q : 0.0f;
+        }
+    };
+    constexpr int NPF = PF > 0 ? PF : 1;
+    float pd[NPF], px[NPF], pq[NPF], pv[NPF], pg[NPF];
+    // where this thread's elements of a chunk lie (token, row) and (token, column): the same for every chunk
+    int rt[NPF], ri[NPF], vt[NPF], vc[NPF];
+#pragma unroll
+    for (int k = 0; k < NPF; ++k) {
+        const int e = tid + k * SCAN_THREADS;
+        rt[k] = e / Rp;
+        ri[k] = e % Rp;
+        vt[k] = e >> cl_shift;
+        vc[k] = e & (CL - 1);
+    }
+    float* gates = part + SCAN_CHUNK * SCAN_THREADS;  // [CHUNK][CL] (wkv): silu of the gate's logits
+    auto fetch = [&](int from) {  // (past the request's last token: its last token once more, never staged)
+        const int c0 = min(from, end - 1);
+        const int len = min(SCAN_CHUNK, end - c0);
+#pragma unroll
+        for (int k = 0; k < NPF; ++k) {
+            raw_rows(c0, len, rt[k], ri[k], pd[k], px[k], pq[k]);
+            pv[k] = raw_val(c0, len, vt[k], vc[k]);
+            if (MODE == 0) pg[k] = raw_gate(c0, len, vt[k], vc[k]);
+        }
+    };
+    if (PF > 0) fetch(begin);
 
     for (int c0 = begin; c0 < end; c0 += SCAN_CHUNK) {
         const int len = min(SCAN_CHUNK, end - c0);
         __syncthreads();  // the chunk before has been read
-        for (int e = tid; e < len * Rp; e += SCAN_THREADS) {
-            const int tt = e / Rp, i = e % Rp;
-            const int64_t t = c0 + tt;
-            float d = 0.0f, x = 0.0f, q = 0.0f;
-            if (i < R) {
-                if (MODE == 0) {
-                    const int64_t at = t * a.ld + h * R + i;
-                    d = expf(-expf(a.wraw[at] + a.w0[h * R + i]));
-                    x = a.k[at];
-                    q = a.r[at];
-                } else {
-                    const float dt = softplus_f(a.dtraw[t * a.ldp + h] + a.dt_bias[h]);
-                    d = expf(neg_A * dt);
-                    x = dt * a.xbc[t * a.ldx + a.inner + g * R + i];
-                    q = a.xbc[t * a.ldx + a.inner + a.G * R + g * R + i];
+        if (PF > 0) {
+#pragma unroll
+            for (int k = 0; k < NPF; ++k) {
+                put_rows(len, rt[k], ri[k], pd[k], px[k], pq[k]);
+                if (vt[k] < len) {
+                    val[vt[k] * CL + vc[k]] = vc[k] < C ? pv[k] : 0.0f;
+                    if (MODE == 0) gates[vt[k] * CL + vc[k]] = silu_f(pg[k]);
                 }
             }
-            decay[e] = d;
-            inr[e] = x;
-            qr[e] = q;
-        }
-        for (int e = tid; e < len * CL; e += SCAN_THREADS) {
-            const int tt = e / CL, jj = e % CL;
-            const int64_t t = c0 + tt;
-            float x = 0.0f;
-            if (jj < C) x = MODE == 0 ? a.v[t * a.ld + h * C + jj] : a.xbc[t * a.ldx + h * C + jj];
-            val[e] = x;
+        } else {
+            for (int e = tid; e < len * Rp; e += SCAN_THREADS) {
+                float d, x, q;
+                raw_rows(c0, len, e / Rp, e % Rp, d, x, q);
+                put_rows(len, e / Rp, e % Rp, d, x, q);
+            }
+            for (int e = tid; e < len * CL; e += SCAN_THREADS) {
+                val[e] = (e & (CL - 1)) < C ? raw_val(c0, len, e >> cl_shift, e & (CL - 1)) : 0.0f;
+                if (MODE == 0) gates[e] = silu_f(raw_gate(c0, len, e >> cl_shift, e & (CL - 1)));
+            }
         }
         __syncthreads();
+        if (PF > 0) fetch(c0 + SCAN_CHUNK);  // on their way while this chunk is computed
+#pragma unroll 2
         for (int tt = 0; tt < len; ++tt) {
             const float vj = val[tt * CL + j];
-            const float* dr = decay + tt * Rp + i0;
-            const float* ir = inr + tt * Rp + i0;
-            const float* qq = qr + tt * Rp + i0;
+            const float4* dr = reinterpret_cast<const float4*>(decay + tt * Rp + i0);
+            const float4* ir = reinterpret_cast<const float4*>(inr + tt * Rp + i0);
+            const float4* qq = reinterpret_cast<const float4*>(qr + tt * Rp + i0);
             float acc = 0.0f;
 #pragma unroll
-            for (int ii = 0; ii < REG; ++ii) {
-                if (ii < a.rows_per) {
-                    const float kin = ir[ii] * vj;
-                    if (MODE == 0) {
-                        acc = fmaf(qq[ii], fmaf(bonus[i0 + ii], kin, S[ii]), acc);
-                        S[ii] = fmaf(dr[ii], S[ii], kin);
-                    } else {
-                        S[ii] = fmaf(dr[ii], S[ii], kin);
-                        acc = fmaf(qq[ii], S[ii], acc);
+            for (int i4 = 0; i4 < REG / 4; ++i4) {
+                if (4 * i4 < a.rows_per) {
+                    const float4 d4 = dr[i4], k4 = ir[i4], q4 = qq[i4];
+                    const float dd[4] = {d4.x, d4.y, d4.z, d4.w}, kk[4] = {k4.x, k4.y, k4.z, k4.w}, qv[4] = {q4.x, q4.y, q4.z, q4.w};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int ii = 4 * i4 + e;
+                        const float kin = kk[e] * vj;
+                        if (MODE == 0) {
+                            acc = fmaf(qv[e], fmaf(bonus[ii], kin, S[ii]), acc);
+                            S[ii] = fmaf(dd[e], S[ii], kin);
+                        } else {
+                            S[ii] = fmaf(dd[e], S[ii], kin);
+                            acc = fmaf(qv[e], S[ii], acc);
+                        }
                     }
                 }
             }
@@ -173,13 +240,14 @@ scan_kernel(ScanArgs a) {
                     float o = 0.0f;
                     for (int b = 0; b < n_rb; ++b) o += part[(tt * n_rb + b) * CL + jj];
                     const int col = h * C + jj;
-                    const float y = o * rinv * a.norm_w[col] * silu_f(a.gate[t * a.ld + col]);
+                    const float y = o * rinv * a.norm_w[col] * gates[tt * CL + jj];
                     static_cast<OutT*>(a.out)[t * (static_cast<int64_t>(a.H) * C) + col] = from_float<OutT>(y);
                 }
             }
         } else {
-            for (int e = tid; e < len * C; e += SCAN_THREADS) {
-                const int tt = e / C, jj = e % C;
+            for (int e = tid; e < len * CL; e += SCAN_THREADS) {
+                const int tt = e >> cl_shift, jj = e & (CL - 1);
+                if (jj >= C) continue;
                 float o = 0.0f;
                 for (int b = 0; b < n_rb; ++b) o += part[(tt * n_rb + b) * CL + jj];
                 static_cast<float*>(a.out)[(c0 + tt) * a.ldy + h * C + jj] = fmaf(dskip, val[tt * CL + jj], o);
@@ -207,32 +275,43 @@ scan_kernel(ScanArgs a) {
     }
 }
 
-// rows a thread holds, lanes side by side, and the dynamic LDS for a state of rows x cols; false when
-// the kernel does not take the size
-static bool scan_shape(int rows, int cols, int* col_lanes, int* rows_per, int* reg, size_t* smem) {
+// rows a thread holds (a multiple of 4), lanes side by side, elements a thread fetches ahead, and the dynamic LDS for a
+// state of rows x cols; false when the kernel does not take the size
+static bool scan_shape(int rows, int cols, int* col_lanes, int* rows_per, int* reg, int* pf, size_t* smem) {
     if (rows <= 0 || cols <= 0 || cols > SCAN_THREADS) return false;
     int cl = 1;
     while (cl < cols) cl *= 2;
+    // no more blocks of rows than the rows fill four at a time (few columns of many rows: lanes idle rather than rows staged as zeros)
+    while (SCAN_THREADS / cl > 1 && (SCAN_THREADS / cl) * 4 > (rows + 3) / 4 * 4) cl *= 2;
     const int n_rb = SCAN_THREADS / cl;
-    const int rp = (rows + n_rb - 1) / n_rb;
+    const int rp = ((rows + n_rb - 1) / n_rb + 3) / 4 * 4;
     if (rp > 64) return false;
     *col_lanes = cl;
     *rows_per = rp;
     *reg = rp <= 8 ? 8 : rp <= 16 ? 16 : rp <= 32 ? 32 : 64;
     const int Rp = n_rb * rp;
-    *smem = sizeof(float) * (static_cast<size_t>(3) * SCAN_CHUNK * Rp + SCAN_CHUNK * cl + SCAN_CHUNK * SCAN_THREADS + Rp);
+    const int ahead = (SCAN_CHUNK * (Rp > cl ? Rp : cl) + SCAN_THREADS - 1) / SCAN_THREADS;
+    *pf = ahead <= 4 ? 4 : ahead <= 8 ? 8 : 0;
+    *smem = sizeof(float) * (static_cast<size_t>(3) * SCAN_CHUNK * Rp + 2 * SCAN_CHUNK * cl + SCAN_CHUNK * SCAN_THREADS);
     return *smem <= 64 * 1024;
 }
 
-template <int MODE, typename OutT>
-static void launch_scan(const ScanArgs& a, int n_seqs, int reg, size_t smem, hipStream_t stream) {
+template <int MODE, typename OutT, int PF>
+static void launch_scan_pf(const ScanArgs& a, int n_seqs, int reg, size_t smem, hipStream_t stream) {
     dim3 grid(n_seqs, a.H);
     switch (reg) {
-        case 8: scan_kernel<MODE, 8, OutT><<<grid, SCAN_THREADS, smem, stream>>>(a); break;
-        case 16: scan_kernel<MODE, 16, OutT><<<grid, SCAN_THREADS, smem, stream>>>(a); break;
-        case 32: scan_kernel<MODE, 32, OutT><<<grid, SCAN_THREADS, smem, stream>>>(a); break;
-        default: scan_kernel<MODE, 64, OutT><<<grid, SCAN_THREADS, smem, stream>>>(a); break;
+        case 8: scan_kernel<MODE, 8, PF, OutT><<<grid, SCAN_THREADS, smem, stream>>>(a); break;
+        case 16: scan_kernel<MODE, 16, PF, OutT><<<grid, SCAN_THREADS, smem, stream>>>(a); break;
+        case 32: scan_kernel<MODE, 32, PF, OutT><<<grid, SCAN_THREADS, smem, stream>>>(a); break;
+        default: scan_kernel<MODE, 64, PF, OutT><<<grid, SCAN_THREADS, smem, stream>>>(a); break;
     }
+}
+
+template <int MODE, typename OutT>
+static void launch_scan(const ScanArgs& a, int n_seqs, int reg, int pf, size_t smem, hipStream_t stream) {
+    if (pf == 4) launch_scan_pf<MODE, OutT, 4>(a, n_seqs, reg, smem, stream);
+    else if (pf == 8) launch_scan_pf<MODE, OutT, 8>(a, n_seqs, reg, smem, stream);
+    else launch_scan_pf<MODE, OutT, 0>(a, n_seqs, reg, smem, stream);
 }
 
 template <typename T>
@@ -314,9 +393,9 @@ gated_group_norm_kernel(T* __restrict__ out, const float* __restrict__ y, int64_
 using namespace liyab;
 
 extern "C" int liyab_scan_takes(int rows, int cols) {
-    int cl, rp, reg;
+    int cl, rp, reg, pf;
     size_t smem;
-    return scan_shape(rows, cols, &cl, &rp, &reg, &smem) ? 1 : 0;
+    return scan_shape(rows, cols, &cl, &rp, &reg, &pf, &smem) ? 1 : 0;
 }
 
 extern "C" int liyab_wkv_scan(void* out, int out_dtype, const float* r, const float* k, const float* v, const float* wraw, const float* gate,
@@ -332,16 +411,16 @@ extern "C" int liyab_wkv_scan(void* out, int out_dtype, const float* r, const fl
                   "wkv_scan: a slot of %lld floats does not hold the state", static_cast<long long>(state_stride));
     ScanArgs a = {};
     size_t smem;
-    int reg;
-    LIYAB_REQUIRE(scan_shape(D, D, &a.col_lanes, &a.rows_per, &reg, &smem), "wkv_scan: heads of %d are not taken", D);
+    int reg, pf;
+    LIYAB_REQUIRE(scan_shape(D, D, &a.col_lanes, &a.rows_per, &reg, &pf, &smem), "wkv_scan: heads of %d are not taken", D);
     if (n_seqs == 0) return 0;
     a.state = state; a.state_stride = state_stride; a.n_slots = n_slots;
     a.seq_starts = seq_starts; a.positions = positions; a.state_slots = state_slots;
     a.H = H; a.rows = D; a.cols = D;
     a.keep_src = keep_src; a.keep_bf16 = keep_dtype == kBF16; a.keep_ld = keep_ld; a.keep_width = keep_width; a.keep_ring = 1; a.keep_off = keep_off;
     a.r = r; a.k = k; a.v = v; a.wraw = wraw; a.gate = gate; a.ld = ld; a.w0 = w0; a.u = u; a.norm_w = norm_w; a.eps = eps; a.out = out;
-    if (out_dtype == kF32) launch_scan<0, float>(a, n_seqs, reg, smem, stream);
-    else if (out_dtype == kBF16) launch_scan<0, bf16_t>(a, n_seqs, reg, smem, stream);
+    if (out_dtype == kF32) launch_scan<0, float>(a, n_seqs, reg, pf, smem, stream);
+    else if (out_dtype == kBF16) launch_scan<0, bf16_t>(a, n_seqs, reg, pf, smem, stream);
     else return fail(1, "wkv_scan: unknown dtype %d", out_dtype);
     return check_launch("wkv_scan");
 }
@@ -358,8 +437,8 @@ extern "C" int liyab_ssd_scan(float* y, int64_t ldy, const float* xbc, int64_t l
                   "ssd_scan: a slot of %lld floats does not hold the state", static_cast<long long>(state_stride));
     ScanArgs a = {};
     size_t smem;
-    int reg;
-    LIYAB_REQUIRE(scan_shape(N, P, &a.col_lanes, &a.rows_per, &reg, &smem), "ssd_scan: a state of %d x %d a head is not taken", N, P);
+    int reg, pf;
+    LIYAB_REQUIRE(scan_shape(N, P, &a.col_lanes, &a.rows_per, &reg, &pf, &smem), "ssd_scan: a state of %d x %d a head is not taken", N, P);
     if (n_seqs == 0) return 0;
     a.state = state; a.state_stride = state_stride; a.n_slots = n_slots;
     a.seq_starts = seq_starts; a.positions = positions; a.state_slots = state_slots;
@@ -367,7 +446,7 @@ extern "C" int liyab_ssd_scan(float* y, int64_t ldy, const float* xbc, int64_t l
     a.keep_src = keep_src; a.keep_bf16 = 0; a.keep_ld = keep_ld; a.keep_width = keep_width; a.keep_ring = keep_ring; a.keep_off = keep_off;
     a.out = y; a.ldy = ldy; a.xbc = xbc; a.ldx = ldx; a.dtraw = dtraw; a.ldp = ldp; a.dt_bias = dt_bias; a.A_log = A_log; a.Dskip = Dskip;
     a.G = G; a.inner = static_cast<int>(inner);
-    launch_scan<1, float>(a, n_seqs, reg, smem, stream);
+    launch_scan<1, float>(a, n_seqs, reg, pf, smem, stream);
     return check_launch("ssd_scan");
 }
 

@@ -1331,10 +1331,12 @@ def scan_takes(rows: int, cols: int) -> bool:
     lanes = 1
     while lanes < cols:
         lanes *= 2
+    while 256 // lanes > 1 and (256 // lanes) * 4 > -(-rows // 4) * 4:
+        lanes *= 2
     blocks = 256 // lanes
-    per = -(-rows // blocks)
+    per = -(-(-(-rows // blocks)) // 4) * 4  # (rows a thread: a multiple of 4)
     staged = blocks * per
-    return per <= 64 and 4 * (3 * 16 * staged + 16 * lanes + 16 * 256 + staged) <= 64 * 1024
+    return per <= 64 and 4 * (3 * 16 * staged + 2 * 16 * lanes + 16 * 256) <= 64 * 1024
 
 
 def _step_lists(ctx, n: int) -> None:
