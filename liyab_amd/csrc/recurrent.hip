@@ -17,7 +17,8 @@
 // taps - 1 inputs of a short convolution), at ring place position % ring: after every read of them, since
 // the kernels that read them ran before this one.
 //
-// liyab_token_shift: m_c[t] = h[t] + (h[t - 1] - h[t]) * mu_c for each of n_mix learned mixes, the previous
+// liyab_token_shift: m_c[t] = h[t] + (h[t - 1] - h[t]) * mu_c for each of n_mix learned mixes (a token's mixes side by side
+//   in its row of the output, [n, n_mix * d]), the previous
 //   row taken from the step's rows, from the request's slot, or zero at position 0.
 // liyab_conv_act: out[t, c] = silu(bias[c] + sum_j w[c, j] * in[t - taps + 1 + j, c]) over a request's
 //   own rows in time (the last column of w is the current row's), earlier rows from the ring.
@@ -331,7 +332,7 @@ token_shift_kernel(T* __restrict__ out, const T* __restrict__ h, const float* __
         if (p > 0) prev = from_step ? to_float<T>(h[static_cast<int64_t>(t - 1) * d + i]) : (from_state ? prev_state[i] : 0.0f);
         const float diff = prev - cur;
         for (int c = 0; c < n_mix; ++c)
-            out[(static_cast<int64_t>(c) * n + t) * d + i] = from_float<T>(fmaf(diff, mu[c * d + i], cur));
+            out[(static_cast<int64_t>(t) * n_mix + c) * d + i] = from_float<T>(fmaf(diff, mu[c * d + i], cur));
     }
 }
 

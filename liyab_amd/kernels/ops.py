@@ -1354,14 +1354,14 @@ def _state(state: torch.Tensor, what: str) -> int:
 
 
 def token_shift(out: torch.Tensor, h: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, prev_off: int, ctx) -> None:
-    """out[c, t] = h[t] + (h[t - 1] - h[t]) * mu[c]; h [n, d] in the compute dtype, mu float32 [n_mix, d], out [n_mix, n, d];
+    """out[t, c] = h[t] + (h[t - 1] - h[t]) * mu[c]; h [n, d] in the compute dtype, mu float32 [n_mix, d], out [n, n_mix, d];
     the row before a request's first row of the step is state[slot, prev_off : prev_off + d], zeros at position 0."""
     _dev(out, "out")
     _dev(h, "h")
     n, d = h.shape
     stride = _state(state, "token_shift")
-    if not h.is_contiguous() or not out.is_contiguous() or out.dtype != h.dtype or mu.dim() != 2 or tuple(out.shape) != (mu.shape[0], n, d):
-        raise KernelError("token_shift: h [n, d] and out [n_mix, n, d] must be contiguous and of one dtype")
+    if not h.is_contiguous() or not out.is_contiguous() or out.dtype != h.dtype or mu.dim() != 2 or tuple(out.shape) != (n, mu.shape[0], d):
+        raise KernelError("token_shift: h [n, d] and out [n, n_mix, d] must be contiguous and of one dtype")
     _f32vec(mu, "mu", mu.shape[0] * d)
     if prev_off < 0 or prev_off + d > stride or ctx.n_tokens != n:
         raise KernelError("token_shift: the previous row does not lie in the slot, or h is not the step's rows")

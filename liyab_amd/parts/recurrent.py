@@ -25,6 +25,7 @@ class WKV:
     takes_padding_rows = True  # (the recurrence walks the requests' own rows; rows behind them are computed by the products only)
 
     MIXES = ("r", "k", "v", "g", "w")
+    GROUPED_ROWS = 128  # steps of up to this many rows run the four products as one grouped launch
 
     def __init__(self, spec, store, dtype: torch.dtype):
         self.dtype = dtype
@@ -34,7 +35,8 @@ class WKV:
             raise Unsupported(f"wkv: heads of {D} are not supported")
         t = spec.tensors
         self.mu = store.fetch_joined([t["mu_" + c] for c in self.MIXES], [(d,)] * 5, "vector", "stack")
-        self.weights = [store.fetch(t[c], (H * D, d), "matrix") for c in ("r", "k", "v", "g")]
+        # receptance, key, value and gate: one matrix a mix, stacked, so that steps of few rows run them as one launch
+        self.weights = store.fetch_joined([t[c] for c in ("r", "k", "v", "g")], [(H * D, d)] * 4, "matrix", "stack")
         self.w1 = store.fetch(t["w1"], (R, d), "matrix")
         self.w2 = store.fetch(t["w2"], (H * D, R), "matrix")
         self.w0 = store.fetch(t["w0"], (H * D,), "vector")
@@ -52,13 +54,19 @@ class WKV:
                 out: Optional[torch.Tensor] = None):
         h = as_tensor(h)
         n, ws, HD = h.shape[0], ctx.workspace, self.n_head * self.head_dim
-        mixes = ws.get("wkv_mixes", (5, n, self.width), self.dtype)
+        d = self.width
+        mixes = ws.get("wkv_mixes", (n, 5, d), self.dtype)
         ops.token_shift(mixes, h, self.mu, state, HD * self.head_dim, ctx)
+        mixes = mixes.view(n, 5 * d)
         proj = ws.get("wkv_proj", (n, 5 * HD), torch.float32)
-        for c, w in enumerate(self.weights):
-            linear(mixes[c], w, None, out=proj[:, c * HD:(c + 1) * HD])
+        if n <= self.GROUPED_ROWS:
+            # four products of four inputs in one launch (a step of few rows is a chain of launches, not of bytes)
+            ops.heads_product(proj[:, :4 * HD], mixes[:, :4 * d], self.weights)
+        else:
+            for c in range(4):
+                linear(mixes[:, c * d:(c + 1) * d], self.weights[c], None, out=proj[:, c * HD:(c + 1) * HD])
         low = ws.get("wkv_low", (n, self.rank), torch.float32)
-        linear(mixes[4], self.w1, None, out=low)
+        linear(mixes[:, 4 * d:], self.w1, None, out=low)
         low_act = ws.get("wkv_low_act", (n, self.rank), self.dtype)
         ops.activate(low_act, low, "tanh")
         linear(low_act, self.w2, None, out=proj[:, 4 * HD:])
@@ -108,11 +116,13 @@ class StateSpace:
         return StateSpec((self.inner * self.n_state + (self.taps - 1) * self.channels,))
 
     def forward(self, h, ctx: StepContext, cache, state, residual: Optional[torch.Tensor], writes_cache: bool = True,
-                out: Optional[torch.Tensor] = None):
+                out: Optional[torch.Tensor] = None, proj: Optional[torch.Tensor] = None):
+        """`proj`: the input projection's 32-bit rows, when the caller has made them (as columns of a wider product)."""
         h = as_tensor(h)
         n, ws, inner, C = h.shape[0], ctx.workspace, self.inner, self.channels
-        proj = ws.get("ssm_in", (n, self.in_weight.shape[0]), torch.float32)
-        linear(h, self.in_weight, None, out=proj)
+        if proj is None:
+            proj = ws.get("ssm_in", (n, self.in_weight.shape[0]), torch.float32)
+            linear(h, self.in_weight, None, out=proj)
         raw = proj[:, inner:inner + C]
         xbc = ws.get("ssm_xbc", (n, C), torch.float32)
         ops.conv_act(xbc, raw, self.conv, self.conv_bias, state, inner * self.n_state, ctx)

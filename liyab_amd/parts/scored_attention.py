@@ -121,13 +121,15 @@ class ScoredAttention:
         return None
 
     def forward(self, h, ctx: StepContext, cache: LayerCache, state, residual: Optional[torch.Tensor],
-                writes_cache: bool = True, out: Optional[torch.Tensor] = None):
-        """Adds the mixer's result into `residual`, or, with `out` (float32 [n, width]), leaves it there."""
+                writes_cache: bool = True, out: Optional[torch.Tensor] = None, proj: Optional[torch.Tensor] = None):
+        """Adds the mixer's result into `residual`, or, with `out` (float32 [n, width]), leaves it there. `proj`: the input
+        projection's 32-bit rows, when the caller has made them (as columns of a wider product)."""
         h = as_tensor(h)
         n, ws, H, D, V = h.shape[0], ctx.workspace, self.n_head, self.head_dim, self.value_dim
         group = ctx.groups[cache.group]
-        proj = ws.get("scored_in", (n, self.in_weight.shape[0]), torch.float32)
-        linear(h, self.in_weight, None, out=proj)
+        if proj is None:
+            proj = ws.get("scored_in", (n, self.in_weight.shape[0]), torch.float32)
+            linear(h, self.in_weight, None, out=proj)
         q = ws.get("scored_q", (n, H * D), self.dtype)
         if not writes_cache:
             raise Unsupported("scored attention: a run that reads another run's cache is not supported")

@@ -8,6 +8,7 @@ import torch
 
 from ..kernels import ops
 from .base import StepContext, settled
+from .linear import linear
 from .norms import as_tensor
 from .registry import build_part, register_mixer
 
@@ -39,6 +40,14 @@ class SideBySide:
         t = spec.tensors
         self.left_out = store.fetch(t["left_out"], (self.width,), "vector")
         self.right_out = store.fetch(t["right_out"], (self.width,), "vector")
+        # both read the same rows: where both have one input projection and take its rows from the caller (`in_weight`,
+        # forward(..., proj=)), the two run as one product [left | right]
+        self.joint_weight = None
+        if all(isinstance(getattr(p, "in_weight", None), torch.Tensor) and "proj" in p.forward.__code__.co_varnames for p in (self.left, self.right)) \
+                and self.left.in_weight.dtype == self.right.in_weight.dtype:
+            lw, rw = self.left.in_weight, self.right.in_weight
+            self.joint_weight = store.derived(("joined_rows", id(lw), id(rw)), lambda: torch.cat([lw, rw], dim=0).contiguous())
+            self.left_cols = lw.shape[0]
         planners = [p for p in (getattr(self.left, "step_planner", None), getattr(self.right, "step_planner", None)) if p is not None]
         if len(planners) > 1:
             raise ValueError("mixers side by side: only one of them may plan a step")
@@ -57,8 +66,14 @@ class SideBySide:
         n, ws = h.shape[0], ctx.workspace
         a = ws.get("side_left", (n, self.width), torch.float32)
         b = ws.get("side_right", (n, self.width), torch.float32)
-        self.left.forward(h, ctx, cache, state, None, writes_cache=writes_cache, out=a)
-        self.right.forward(h, ctx, cache, state, None, writes_cache=writes_cache, out=b)
+        if self.joint_weight is not None:
+            proj = ws.get("side_in", (n, self.joint_weight.shape[0]), torch.float32)
+            linear(h, self.joint_weight, None, out=proj)
+            self.left.forward(h, ctx, cache, state, None, writes_cache=writes_cache, out=a, proj=proj[:, :self.left_cols])
+            self.right.forward(h, ctx, cache, state, None, writes_cache=writes_cache, out=b, proj=proj[:, self.left_cols:])
+        else:
+            self.left.forward(h, ctx, cache, state, None, writes_cache=writes_cache, out=a)
+            self.right.forward(h, ctx, cache, state, None, writes_cache=writes_cache, out=b)
         if out is not None:
             ops.fill_(out, 0)
             ops.mean_norm_add(out, a, b, self.left_out, self.right_out, self.eps, self.weight)
