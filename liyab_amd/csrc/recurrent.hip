@@ -29,8 +29,9 @@
 
 namespace liyab {
 
-constexpr int SCAN_THREADS = 256;
+constexpr int SCAN_THREADS = 512;  // eight waves, two a SIMD: one wave's waits for LDS and for its own results hide behind the other's work
 constexpr int SCAN_CHUNK = 16;  // tokens staged through LDS together
+constexpr size_t SCAN_MAX_LDS = 128 * 1024;
 
 __device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z)); }
 __device__ __forceinline__ float softplus_f(float z) { return z > 20.0f ? z : log1pf(expf(z)); }
@@ -196,22 +197,46 @@ scan_kernel(ScanArgs a) {
         }
         __syncthreads();
         if (PF > 0) fetch(c0 + SCAN_CHUNK);  // on their way while this chunk is computed
-#pragma unroll 2
-        for (int tt = 0; tt < len; ++tt) {
-            const float vj = val[tt * CL + j];
+        // A token's operands are asked for while the token before is computed: the reads of LDS stand ahead of the store of
+        // the partial sums in the program's order (the compiler cannot move them past it by itself), and with one wave a SIMD
+        // nothing else hides their way.
+        float4 nd[REG / 4], nk[REG / 4], nq[REG / 4];
+        float nv;
+        auto operands = [&](int tt) {
+            nv = val[tt * CL + j];
             const float4* dr = reinterpret_cast<const float4*>(decay + tt * Rp + i0);
             const float4* ir = reinterpret_cast<const float4*>(inr + tt * Rp + i0);
             const float4* qq = reinterpret_cast<const float4*>(qr + tt * Rp + i0);
-            float acc = 0.0f;
+#pragma unroll
+            for (int i4 = 0; i4 < REG / 4; ++i4) {
+                const int at = 4 * i4 < a.rows_per ? i4 : 0;  // (rows this thread does not hold: its first four once more)
+                nd[i4] = dr[at];
+                nk[i4] = ir[at];
+                nq[i4] = qq[at];
+            }
+        };
+        operands(0);
+        for (int tt = 0; tt < len; ++tt) {
+            float4 cd[REG / 4], ck[REG / 4], cq[REG / 4];
+            const float vj = nv;
+#pragma unroll
+            for (int i4 = 0; i4 < REG / 4; ++i4) {
+                cd[i4] = nd[i4];
+                ck[i4] = nk[i4];
+                cq[i4] = nq[i4];
+            }
+            operands(min(tt + 1, len - 1));
+            float acc0 = 0.0f, acc1 = 0.0f;
 #pragma unroll
             for (int i4 = 0; i4 < REG / 4; ++i4) {
                 if (4 * i4 < a.rows_per) {
-                    const float4 d4 = dr[i4], k4 = ir[i4], q4 = qq[i4];
-                    const float dd[4] = {d4.x, d4.y, d4.z, d4.w}, kk[4] = {k4.x, k4.y, k4.z, k4.w}, qv[4] = {q4.x, q4.y, q4.z, q4.w};
+                    const float dd[4] = {cd[i4].x, cd[i4].y, cd[i4].z, cd[i4].w}, kk[4] = {ck[i4].x, ck[i4].y, ck[i4].z, ck[i4].w},
+                                qv[4] = {cq[i4].x, cq[i4].y, cq[i4].z, cq[i4].w};
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         const int ii = 4 * i4 + e;
                         const float kin = kk[e] * vj;
+                        float& acc = e % 2 ? acc1 : acc0;
                         if (MODE == 0) {
                             acc = fmaf(qv[e], fmaf(bonus[ii], kin, S[ii]), acc);
                             S[ii] = fmaf(dd[e], S[ii], kin);
@@ -222,7 +247,7 @@ scan_kernel(ScanArgs a) {
                     }
                 }
             }
-            part[(tt * n_rb + rb) * CL + j] = acc;
+            part[(tt * n_rb + rb) * CL + j] = acc0 + acc1;
         }
         __syncthreads();
         if (MODE == 0) {
@@ -294,17 +319,26 @@ static bool scan_shape(int rows, int cols, int* col_lanes, int* rows_per, int* r
     const int ahead = (SCAN_CHUNK * (Rp > cl ? Rp : cl) + SCAN_THREADS - 1) / SCAN_THREADS;
     *pf = ahead <= 4 ? 4 : ahead <= 8 ? 8 : 0;
     *smem = sizeof(float) * (static_cast<size_t>(3) * SCAN_CHUNK * Rp + 2 * SCAN_CHUNK * cl + SCAN_CHUNK * SCAN_THREADS);
-    return *smem <= 64 * 1024;
+    return *smem <= SCAN_MAX_LDS;
+}
+
+template <int MODE, int REG, int PF, typename OutT>
+static void launch_scan_one(const ScanArgs& a, int n_seqs, size_t smem, hipStream_t stream) {
+    auto kern = scan_kernel<MODE, REG, PF, OutT>;
+    if (smem > 48 * 1024) {
+        static bool allowed = false;  // (once a kernel: more dynamic LDS than the default limit)
+        if (!allowed) allowed = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(SCAN_MAX_LDS)) == hipSuccess;
+    }
+    kern<<<dim3(n_seqs, a.H), SCAN_THREADS, smem, stream>>>(a);
 }
 
 template <int MODE, typename OutT, int PF>
 static void launch_scan_pf(const ScanArgs& a, int n_seqs, int reg, size_t smem, hipStream_t stream) {
-    dim3 grid(n_seqs, a.H);
     switch (reg) {
-        case 8: scan_kernel<MODE, 8, PF, OutT><<<grid, SCAN_THREADS, smem, stream>>>(a); break;
-        case 16: scan_kernel<MODE, 16, PF, OutT><<<grid, SCAN_THREADS, smem, stream>>>(a); break;
-        case 32: scan_kernel<MODE, 32, PF, OutT><<<grid, SCAN_THREADS, smem, stream>>>(a); break;
-        default: scan_kernel<MODE, 64, PF, OutT><<<grid, SCAN_THREADS, smem, stream>>>(a); break;
+        case 8: launch_scan_one<MODE, 8, PF, OutT>(a, n_seqs, smem, stream); break;
+        case 16: launch_scan_one<MODE, 16, PF, OutT>(a, n_seqs, smem, stream); break;
+        case 32: launch_scan_one<MODE, 32, PF, OutT>(a, n_seqs, smem, stream); break;
+        default: launch_scan_one<MODE, 64, PF, OutT>(a, n_seqs, smem, stream); break;
     }
 }
 

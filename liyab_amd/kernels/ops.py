@@ -1325,18 +1325,19 @@ def mean_norm_add(x: torch.Tensor, a: torch.Tensor, b: torch.Tensor, wa: torch.T
 # -- mixers with a matrix of state a head ---------------------------------------------------------------
 def scan_takes(rows: int, cols: int) -> bool:
     """Whether the recurrence kernel takes a state of rows x cols a head (csrc/recurrent.hip: scan_shape): a column a
-    thread, up to 64 rows of it in registers, sixteen tokens' vectors staged in at most 64 KiB of LDS."""
-    if rows <= 0 or not 0 < cols <= 256:
+    thread of 512, up to 64 rows of it in registers (a multiple of 4), sixteen tokens' vectors staged in at most 128 KiB of LDS."""
+    threads = 512
+    if rows <= 0 or not 0 < cols <= threads:
         return False
     lanes = 1
     while lanes < cols:
         lanes *= 2
-    while 256 // lanes > 1 and (256 // lanes) * 4 > -(-rows // 4) * 4:
+    while threads // lanes > 1 and (threads // lanes) * 4 > -(-rows // 4) * 4:
         lanes *= 2
-    blocks = 256 // lanes
-    per = -(-(-(-rows // blocks)) // 4) * 4  # (rows a thread: a multiple of 4)
+    blocks = threads // lanes
+    per = -(-(-(-rows // blocks)) // 4) * 4
     staged = blocks * per
-    return per <= 64 and 4 * (3 * 16 * staged + 2 * 16 * lanes + 16 * 256) <= 64 * 1024
+    return per <= 64 and 4 * (3 * 16 * staged + 2 * 16 * lanes + 16 * threads) <= 128 * 1024
 
 
 def _step_lists(ctx, n: int) -> None:
