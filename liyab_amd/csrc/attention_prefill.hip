@@ -221,6 +221,9 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
 #pragma unroll
                 for (int z = 0; z < NS; ++z) {
                     const int kb = kb0w + z * AP_KEYS;
+                    // a block that lies at least max_dist behind the wave's earliest query takes the table's last row throughout
+                    const bool far = bias_table != nullptr && pos0 + 32 * qg - (kb + AP_KEYS - 1) >= max_dist;
+                    const float bias_far = bias_table != nullptr ? bias_table[static_cast<int64_t>(max_dist) * n_head + h] : 0.0f;
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
                         float sc = st[z][r] * scale;
@@ -230,8 +233,12 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
                             sc = softcap * (1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + e2));
                         }
                         if (bias_table != nullptr) {
-                            const int kp = kb + 8 * (r / 4) + 4 * g2 + r % 4;
-                            sc += bias_table[static_cast<int64_t>(min(max(qpos - kp, 0), max_dist)) * n_head + h];
+                            if (far) {
+                                sc += bias_far;
+                            } else {
+                                const int kp = kb + 8 * (r / 4) + 4 * g2 + r % 4;
+                                sc += bias_table[static_cast<int64_t>(min(max(qpos - kp, 0), max_dist)) * n_head + h];
+                            }
                         }
                         st[z][r] = sc;
                     }
