@@ -7,7 +7,8 @@
 // each optional); the turning of pairs (2i, 2i + 1) of the first `rot_dims` entries by position * f_i
 // (queries and keys; f from a table); a factor on the query that grows with the logarithm of the
 // position, 1 + coef * ln(floor((p + 1) / every) + 1). Queries go to a dense buffer in the compute type,
-// keys and values to their token's slot of the pages. Norms, angles and factors are 32-bit.
+// keys and values to their token's slot of the pages; the rows they go to may be wider than the heads (dk_out, dv_out),
+// zeros behind them: keys and values padded to one width are what the matrix-core kernels take. Norms, angles and factors are 32-bit.
 //
 // liyab_attention_scored: one workgroup a (token, query head). score = scale * q . k, then, each optional:
 // a soft cap, cap * tanh(score / cap); a learned bias by distance, table[min(i - j, max_dist), head].
@@ -24,8 +25,8 @@ constexpr int AS_THREADS = 256;
 
 template <typename T>
 __global__ void __launch_bounds__(kWave)
-qk_prepare_kernel(const float* __restrict__ src, int64_t ld, int q_off, int k_off, int v_off, int H, int G, int dk, int dv,
-                  T* __restrict__ q_out, T* __restrict__ kc, T* __restrict__ vc, const int* __restrict__ slots, int page_size,
+qk_prepare_kernel(const float* __restrict__ src, int64_t ld, int q_off, int k_off, int v_off, int H, int G, int dk, int dv, int dk_out,
+                  int dv_out, T* __restrict__ q_out, T* __restrict__ kc, T* __restrict__ vc, const int* __restrict__ slots, int page_size,
                   int num_pages, const float* __restrict__ q_norm, const float* __restrict__ k_norm, float eps,
                   const float* __restrict__ freqs, int rot_dims, float temp_coef, int temp_every, const int* __restrict__ positions) {
     const int t = blockIdx.x, hh = blockIdx.y, lane = threadIdx.x;
@@ -46,12 +47,13 @@ qk_prepare_kernel(const float* __restrict__ src, int64_t ld, int q_off, int k_of
         if (is_q && temp_every > 0) temp = 1.0f + temp_coef * logf(static_cast<float>((p + 1) / temp_every) + 1.0f);
         T* dst;
         if (is_q) {
-            dst = q_out + static_cast<int64_t>(t) * H * dk + head * dk;
+            dst = q_out + static_cast<int64_t>(t) * H * dk_out + head * dk_out;
         } else {
             const int64_t slot = slots[t];
             if (slot < 0 || slot >= static_cast<int64_t>(num_pages) * page_size) return;
-            dst = kc + (((slot / page_size) * G + head) * page_size + slot % page_size) * dk;
+            dst = kc + (((slot / page_size) * G + head) * page_size + slot % page_size) * dk_out;
         }
+        for (int i = dk + lane; i < dk_out; i += kWave) dst[i] = from_float<T>(0.0f);  // rows wider than the head: zeros behind it
         // pairs of entries: a lane takes a pair at a time
         for (int i2 = lane; 2 * i2 < dk; i2 += kWave) {
             const int e0 = 2 * i2, e1 = e0 + 1;
@@ -72,8 +74,8 @@ qk_prepare_kernel(const float* __restrict__ src, int64_t ld, int q_off, int k_of
         const int64_t slot = slots[t];
         if (slot < 0 || slot >= static_cast<int64_t>(num_pages) * page_size) return;
         const float* x = row + v_off + head * dv;
-        T* dst = vc + (((slot / page_size) * G + head) * page_size + slot % page_size) * dv;
-        for (int i = lane; i < dv; i += kWave) dst[i] = from_float<T>(x[i]);
+        T* dst = vc + (((slot / page_size) * G + head) * page_size + slot % page_size) * dv_out;
+        for (int i = lane; i < dv_out; i += kWave) dst[i] = from_float<T>(i < dv ? x[i] : 0.0f);
     }
 }
 
@@ -164,13 +166,14 @@ attention_scored_kernel(T* __restrict__ out, int64_t out_stride, const T* __rest
 
 using namespace liyab;
 
-extern "C" int liyab_qk_prepare(const float* src, int64_t ld, int q_off, int k_off, int v_off, int H, int G, int dk, int dv, void* q_out,
-                                void* kc, void* vc, int dtype, const int* slots, int page_size, int num_pages, const float* q_norm,
+extern "C" int liyab_qk_prepare(const float* src, int64_t ld, int q_off, int k_off, int v_off, int H, int G, int dk, int dv, int dk_out,
+                                int dv_out, void* q_out, void* kc, void* vc, int dtype, const int* slots, int page_size, int num_pages, const float* q_norm,
                                 const float* k_norm, float eps, const float* freqs, int rot_dims, float temp_coef, int temp_every,
                                 const int* positions, int n, hipStream_t stream) {
     LIYAB_REQUIRE(src && q_out && kc && vc && slots && positions, "qk_prepare: null pointer");
     LIYAB_REQUIRE(n >= 0 && H > 0 && G > 0 && dk > 0 && dv > 0 && page_size > 0 && num_pages > 0, "qk_prepare: bad sizes");
     LIYAB_REQUIRE(H + 2 * G <= 65535, "qk_prepare: too many heads");
+    LIYAB_REQUIRE(dk_out >= dk && dv_out >= dv, "qk_prepare: rows of %d / %d do not hold heads of %d / %d", dk_out, dv_out, dk, dv);
     LIYAB_REQUIRE(q_off >= 0 && k_off >= 0 && v_off >= 0 && q_off + static_cast<int64_t>(H) * dk <= ld && k_off + static_cast<int64_t>(G) * dk <= ld &&
                       v_off + static_cast<int64_t>(G) * dv <= ld,
                   "qk_prepare: the heads' columns pass the source's rows");
@@ -180,11 +183,11 @@ extern "C" int liyab_qk_prepare(const float* src, int64_t ld, int q_off, int k_o
     dim3 grid(n, H + 2 * G);
     const float* fr = rot_dims > 0 ? freqs : nullptr;
     if (dtype == kF32)
-        qk_prepare_kernel<float><<<grid, kWave, 0, stream>>>(src, ld, q_off, k_off, v_off, H, G, dk, dv, static_cast<float*>(q_out), static_cast<float*>(kc),
+        qk_prepare_kernel<float><<<grid, kWave, 0, stream>>>(src, ld, q_off, k_off, v_off, H, G, dk, dv, dk_out, dv_out, static_cast<float*>(q_out), static_cast<float*>(kc),
                                                              static_cast<float*>(vc), slots, page_size, num_pages, q_norm, k_norm, eps, fr, rot_dims,
                                                              temp_coef, temp_every, positions);
     else if (dtype == kBF16)
-        qk_prepare_kernel<bf16_t><<<grid, kWave, 0, stream>>>(src, ld, q_off, k_off, v_off, H, G, dk, dv, static_cast<bf16_t*>(q_out),
+        qk_prepare_kernel<bf16_t><<<grid, kWave, 0, stream>>>(src, ld, q_off, k_off, v_off, H, G, dk, dv, dk_out, dv_out, static_cast<bf16_t*>(q_out),
                                                               static_cast<bf16_t*>(kc), static_cast<bf16_t*>(vc), slots, page_size, num_pages, q_norm,
                                                               k_norm, eps, fr, rot_dims, temp_coef, temp_every, positions);
     else return fail(1, "qk_prepare: unknown dtype %d", dtype);

@@ -98,7 +98,7 @@ _SIGNATURES = {
     "liyab_token_shift": [P, c_int, P, P, c_int, P, c_int64, c_int, P, P, P, P, c_int, c_int, P],
     "liyab_conv_act": [P, c_int64, P, c_int64, P, P, c_int, P, c_int64, c_int, P, P, P, P, c_int, c_int, P],
     "liyab_gated_group_norm": [P, c_int, P, c_int64, P, c_int64, P, c_float, c_int, c_int, c_int, P],
-    "liyab_qk_prepare": [P, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P, P, P, c_int, P, c_int, c_int, P, P, c_float, P,
+    "liyab_qk_prepare": [P, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P, P, P, c_int, P, c_int, c_int, P, P, c_float, P,
                          c_int, c_float, c_int, P, c_int, P],
     "liyab_attention_scored": [P, c_int64, P, c_int64, P, P, c_int, P, c_int, P, P, c_int, c_float, c_float, c_int, P, c_int, P, c_int64,
                                c_int, c_int, c_int, c_int, c_int, c_int, P],

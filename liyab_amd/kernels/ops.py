@@ -1479,12 +1479,13 @@ def gated_group_norm(out: torch.Tensor, y: torch.Tensor, z: torch.Tensor, weight
 def qk_prepare(src: torch.Tensor, q_out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, slots: torch.Tensor, positions: torch.Tensor,
                *, q_off: int, k_off: int, v_off: int, n_head: int, q_norm: Optional[torch.Tensor] = None, k_norm: Optional[torch.Tensor] = None,
                eps: float = 0.0, freqs: Optional[torch.Tensor] = None, rot_dims: int = 0, temp_coef: float = 0.0, temp_every: int = 0,
-               num_pages: Optional[int] = None) -> None:
+               num_pages: Optional[int] = None, head_dim: Optional[int] = None, value_dim: Optional[int] = None) -> None:
     """From a projection's float32 rows `src` (queries at column q_off, keys at k_off, values at v_off, which may be k_off) to
     queries in `q_out` [n, heads * dk] and keys and values in their slots of the pages (k_cache [pages, kv_heads, page, dk],
     v_cache [.., dv]), all in the compute dtype. Per head, each optional: a root-mean-square norm with a weight [dk] (queries,
     keys), pairs (2i, 2i + 1) of the first rot_dims entries turned by position * freqs[i] (queries, keys), the query times
-    1 + temp_coef * ln(floor((position + 1) / temp_every) + 1). A slot outside the pages is not written."""
+    1 + temp_coef * ln(floor((position + 1) / temp_every) + 1). A slot outside the pages is not written. `head_dim`,
+    `value_dim`: the heads' own widths where the caches' rows (and the queries') are wider, zeros behind the heads."""
     ld = _rows(src, "src")
     n = src.shape[0]
     _dev(q_out, "q_out")
@@ -1492,9 +1493,12 @@ def qk_prepare(src: torch.Tensor, q_out: torch.Tensor, k_cache: torch.Tensor, v_
     _dev(v_cache, "v_cache")
     if k_cache.dim() != 4 or v_cache.dim() != 4 or k_cache.shape[:3] != v_cache.shape[:3] or not k_cache.is_contiguous() or not v_cache.is_contiguous():
         raise KernelError("qk_prepare: caches must be contiguous [pages, kv_heads, page_size, width] with the same pages")
-    _, G, page, dk = k_cache.shape
-    dv = v_cache.shape[3]
-    if src.dtype != torch.float32 or tuple(q_out.shape) != (n, n_head * dk) or not q_out.is_contiguous() or not (q_out.dtype == k_cache.dtype == v_cache.dtype):
+    _, G, page, dk_out = k_cache.shape
+    dv_out = v_cache.shape[3]
+    dk, dv = head_dim or dk_out, value_dim or dv_out
+    if not (0 < dk <= dk_out and 0 < dv <= dv_out):
+        raise KernelError(f"qk_prepare: heads of {dk} / {dv} in rows of {dk_out} / {dv_out}")
+    if src.dtype != torch.float32 or tuple(q_out.shape) != (n, n_head * dk_out) or not q_out.is_contiguous() or not (q_out.dtype == k_cache.dtype == v_cache.dtype):
         raise KernelError("qk_prepare: src must be float32 rows, q_out contiguous [n, heads * dk], queries and caches of one dtype")
     if min(q_off, k_off, v_off) < 0 or q_off + n_head * dk > src.shape[1] or k_off + G * dk > src.shape[1] or v_off + G * dv > src.shape[1]:
         raise KernelError("qk_prepare: the heads' columns pass the source's rows")
@@ -1506,7 +1510,7 @@ def qk_prepare(src: torch.Tensor, q_out: torch.Tensor, k_cache: torch.Tensor, v_
         _f32vec(freqs, "freqs", rot_dims // 2)
     _i32(slots, "slots", n)
     _i32(positions, "positions", n)
-    _lib.call("liyab_qk_prepare", src.data_ptr(), ld, q_off, k_off, v_off, n_head, G, dk, dv, q_out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+    _lib.call("liyab_qk_prepare", src.data_ptr(), ld, q_off, k_off, v_off, n_head, G, dk, dv, dk_out, dv_out, q_out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
               dtype_code(q_out.dtype), slots.data_ptr(), page, _pages(k_cache, num_pages), _ptr(q_norm), _ptr(k_norm), float(eps),
               _ptr(freqs) if rot_dims else None, rot_dims, float(temp_coef), int(temp_every), positions.data_ptr(), n, _stream())
 

@@ -93,6 +93,14 @@ class ScoredAttention:
             at += H * V
         self.in_weight = store.fetch_joined(srcs, shapes, "matrix", "rows")
         self.out_weight = store.fetch(t["out"], (d, H * V), "matrix")
+        # Keys and values of different widths: both planes of the pages as wide as the wider (a multiple of 8), zeros behind the
+        # narrower heads, which is what the engine's paged attention kernels take; zeros in keys and queries add nothing to a
+        # score, zeros in values give zeros in the result, and the output projection gets zero columns for them.
+        self.row_dim = 0
+        if D != V and not self.gated and max(D, V) <= ops.ATTENTION_MAX_HEAD_DIM:
+            P = self.row_dim = -(-max(D, V) // 8) * 8
+            w = self.out_weight
+            self.out_weight = store.derived(("padded_heads", t["out"].name, P), lambda: torch.nn.functional.pad(w.view(d, H, V), (0, P - V)).reshape(d, H * P).contiguous())
         self.q_norm = store.fetch(t["q_norm"], (D,), "vector") if spec.qk_norm else None
         self.k_norm = store.fetch(t["k_norm"], (D,), "vector") if spec.qk_norm else None
         self.rot_dims, self.freqs = 0, None
@@ -115,7 +123,7 @@ class ScoredAttention:
 
     def cache_spec(self) -> Optional[KVSpec]:
         return KVSpec(self.n_kv_head, self.head_dim, self.window,
-                      rows=(("k", self.n_kv_head, self.head_dim), ("v", self.n_kv_head, self.value_dim)))
+                      rows=(("k", self.n_kv_head, self.row_dim or self.head_dim), ("v", self.n_kv_head, self.row_dim or self.value_dim)))
 
     def state_spec(self):
         return None
@@ -130,15 +138,16 @@ class ScoredAttention:
         if proj is None:
             proj = ws.get("scored_in", (n, self.in_weight.shape[0]), torch.float32)
             linear(h, self.in_weight, None, out=proj)
-        q = ws.get("scored_q", (n, H * D), self.dtype)
+        P = self.row_dim
+        q = ws.get("scored_q", (n, H * (P or D)), self.dtype)
         if not writes_cache:
             raise Unsupported("scored attention: a run that reads another run's cache is not supported")
         ops.qk_prepare(proj, q, cache.k, cache.v, group.slots, ctx.positions, q_off=self.q_off, k_off=self.k_off, v_off=self.v_off,
                        n_head=H, q_norm=self.q_norm, k_norm=self.k_norm, eps=self.eps, freqs=self.freqs, rot_dims=self.rot_dims,
-                       temp_coef=self.temp_coef, temp_every=self.temp_every)
-        att = ws.get("scored_att", (n, H * V), self.dtype)
+                       temp_coef=self.temp_coef, temp_every=self.temp_every, head_dim=D, value_dim=V)
+        att = ws.get("scored_att", (n, H * (P or V)), self.dtype)
         gate = proj[:, self.gate_off:self.gate_off + H * V] if self.gated else None
-        if D == V:
+        if D == V or P:
             # keys and values of one width: the paged attention kernels of the engine (tiles of a prompt's queries on the matrix
             # cores, single tokens in splits, the 32-bit form), which cap and bias the scores when asked to
             splits = ops.attention(att, q, cache.k, cache.v, group.block_tables, ctx, n_head=H, scale=self.scale, window=self.window,
