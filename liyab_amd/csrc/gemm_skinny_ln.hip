@@ -43,6 +43,7 @@ struct NormParams {
     const float* weight;  // [K] or null
     const float* bias;    // [K] or null
     float eps;
+    const float* alpha;   // null: LayerNorm. Else the Dynamic Tanh norm, tanh(alpha[0] x) * weight + bias (no statistics)
 };
 
 template <typename OutT, int MAXV, int MT, int NT>
@@ -124,6 +125,23 @@ gemm_skinny_ln_kernel(NormParams ln, const bf16_t* __restrict__ w, int M, int N,
 #pragma unroll
                 for (int j = 0; j < MAXV; ++j)
                     if (q0 + u < ln.n_planes) v[j] += plane[u][j];
+        }
+        if (ln.alpha != nullptr) {
+            // tanh(z) = 1 - 2 / (1 + e^(2z)): one hardware exponential and one reciprocal a value
+            const float a2 = 2.0f * 1.4426950408889634f * ln.alpha[0];
+#pragma unroll
+            for (int j = 0; j < MAXV; ++j)
+                if (keep && lane + kWave * j < nv) {
+                    floatx4 y;
+#pragma unroll
+                    for (int c = 0; c < 4; ++c)
+                        y[c] = (1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(a2 * v[j][c]))) * gw[j][c] + gb[j][c];
+                    uint2 packed;
+                    packed.x = static_cast<uint32_t>(float_to_bf16(y[0])) | (static_cast<uint32_t>(float_to_bf16(y[1])) << 16);
+                    packed.y = static_cast<uint32_t>(float_to_bf16(y[2])) | (static_cast<uint32_t>(float_to_bf16(y[3])) << 16);
+                    *reinterpret_cast<uint2*>(xs + m * ldx + 4 * (lane + kWave * j)) = packed;
+                }
+            return;
         }
         float s = 0.0f;
 #pragma unroll
@@ -267,9 +285,8 @@ using namespace liyab::ln_fold;
 // most 2048. wide: 32 instead of 16 output features a workgroup, for M <= 16 (-1: when
 // there are more strips of 16 than compute units). The residual epilogue
 // is not taken (the product of a norm is never added to the stream as it is).
-extern "C" int liyab_gemm_skinny_ln(const float* planes, int n_planes, int64_t plane_stride, const float* ln_weight,
-                                    const float* ln_bias, float eps, const void* w, int M, int N, int K, int wide,
-                                    const EpiParams* epi_in, hipStream_t stream) {
+static int run_skinny_norm(const float* planes, int n_planes, int64_t plane_stride, const float* ln_weight, const float* ln_bias, float eps,
+                           const float* alpha, const void* w, int M, int N, int K, int wide, const EpiParams* epi_in, hipStream_t stream) {
     LIYAB_REQUIRE(planes && w && epi_in, "gemm_skinny_ln: null operand");
     LIYAB_REQUIRE(M >= 0 && M <= 32 && N > 0 && K > 0, "gemm_skinny_ln: bad sizes M=%d (at most 32) N=%d K=%d", M, N, K);
     LIYAB_REQUIRE(K % 8 == 0 && K <= 2048, "gemm_skinny_ln: K %d must be a multiple of 8, at most 2048", K);
@@ -294,10 +311,24 @@ extern "C" int liyab_gemm_skinny_ln(const float* planes, int n_planes, int64_t p
         wide = (N + 15) / 16 > units ? 1 : 0;
     }
     LIYAB_REQUIRE(!wide || M <= 16, "gemm_skinny_ln: strips of 32 output features go with at most 16 rows (%d)", M);
-    const NormParams ln{planes, n_planes, plane_stride, ln_weight, ln_bias, eps};
+    const NormParams ln{planes, n_planes, plane_stride, ln_weight, ln_bias, eps, alpha};
     if (K <= 256) return launch_ln<1>(ln, w, M, N, K, wide, epi, stream);
     if (K <= 512) return launch_ln<2>(ln, w, M, N, K, wide, epi, stream);
     if (K <= 768) return launch_ln<3>(ln, w, M, N, K, wide, epi, stream);
     if (K <= 1024) return launch_ln<4>(ln, w, M, N, K, wide, epi, stream);
     return launch_ln<8>(ln, w, M, N, K, wide, epi, stream);
+}
+
+extern "C" int liyab_gemm_skinny_ln(const float* planes, int n_planes, int64_t plane_stride, const float* ln_weight,
+                                    const float* ln_bias, float eps, const void* w, int M, int N, int K, int wide,
+                                    const EpiParams* epi_in, hipStream_t stream) {
+    return run_skinny_norm(planes, n_planes, plane_stride, ln_weight, ln_bias, eps, nullptr, w, M, N, K, wide, epi_in, stream);
+}
+
+// The same product over the Dynamic Tanh norm of the rows, tanh(alpha[0] x) * weight + bias (alpha: one float on the device).
+extern "C" int liyab_gemm_skinny_dyt(const float* planes, int n_planes, int64_t plane_stride, const float* weight, const float* bias,
+                                     const float* alpha, const void* w, int M, int N, int K, int wide, const EpiParams* epi_in,
+                                     hipStream_t stream) {
+    LIYAB_REQUIRE(alpha != nullptr, "gemm_skinny_dyt: null operand");
+    return run_skinny_norm(planes, n_planes, plane_stride, weight, bias, 0.0f, alpha, w, M, N, K, wide, epi_in, stream);
 }

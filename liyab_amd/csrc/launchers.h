@@ -44,6 +44,8 @@ int liyab_gemm_att_parts(const float* partials, int n_splits, int n_head, int hd
                          hipStream_t stream);
 int liyab_gemm_skinny_ln(const float* planes, int n_planes, int64_t plane_stride, const float* ln_weight, const float* ln_bias,
                          float eps, const void* w, int M, int N, int K, int wide, const liyab::EpiParams* epi_in, hipStream_t stream);
+int liyab_gemm_skinny_dyt(const float* planes, int n_planes, int64_t plane_stride, const float* weight, const float* bias, const float* alpha,
+                          const void* w, int M, int N, int K, int wide, const liyab::EpiParams* epi_in, hipStream_t stream);
 int liyab_attention_generic(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc, const void* vc, int dtype,
                             const int* block_tables, int max_blocks, const int* tok_seq, const int* tok_pos, int n, float scale,
                             int window, int n_head, int n_kv_head, int hd, int page_size, int num_pages, hipStream_t stream);

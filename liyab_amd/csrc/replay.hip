@@ -83,6 +83,7 @@ static const Entry kEntries[] = {
     LIYAB_ENTRY(liyab_gemm_skinny_parts),
     LIYAB_ENTRY(liyab_gemm_att_parts),
     LIYAB_ENTRY(liyab_gemm_skinny_ln),
+    LIYAB_ENTRY(liyab_gemm_skinny_dyt),
     LIYAB_ENTRY(liyab_attention_generic),
     LIYAB_ENTRY(liyab_attention_decode),
     LIYAB_ENTRY(liyab_attention_merge),

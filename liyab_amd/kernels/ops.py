@@ -651,6 +651,25 @@ def gemm_skinny_ln(x: torch.Tensor, ln_weight: Optional[torch.Tensor], ln_bias: 
               w.data_ptr(), M, w.shape[0], K, wide, ctypes.byref(e), _stream())
 
 
+def gemm_skinny_dyt(x: torch.Tensor, weight: Optional[torch.Tensor], bias: Optional[torch.Tensor], alpha: torch.Tensor, w: torch.Tensor,
+                    out_bias: Optional[torch.Tensor], *, out=None, epilogue: int = EPI_NONE, kv=None, wide: int = -1) -> None:
+    """`gemm_skinny_ln` with the Dynamic Tanh norm in the norm's place: the product over tanh(alpha x) * weight + bias of the
+    float32 rows x [M, K] (alpha: one float32 value on the device)."""
+    ptr, n_parts, stride, M, K = _planes(x, "gemm_skinny_dyt")
+    _dev(w, "w")
+    if w.dtype != torch.bfloat16 or w.dim() != 2 or w.shape[1] != K or not w.is_contiguous():
+        raise KernelError(f"gemm_skinny_dyt: needs contiguous bfloat16 w [N, {K}], got {tuple(w.shape)} {w.dtype}")
+    if not skinny_ln_takes(M, K) or epilogue == EPI_RESIDUAL:
+        raise KernelError(f"gemm_skinny_dyt: {M} rows of {K}, or the residual epilogue, are outside what it takes")
+    _f32vec(weight, "norm weight", K)
+    _f32vec(bias, "norm bias", K)
+    _f32vec(alpha, "norm alpha", 1)
+    e = _epilogue(_Rows(M, torch.bfloat16), w, out_bias, out, None, epilogue, kv)
+    e.exact = 0
+    _lib.call("liyab_gemm_skinny_dyt", ptr, n_parts, stride, _ptr(weight), _ptr(bias), alpha.data_ptr(), w.data_ptr(), M, w.shape[0], K, wide,
+              ctypes.byref(e), _stream())
+
+
 def skinny_ln_takes(M: int, K: int) -> bool:
     """What the product kernel with the norm inside takes: one or two tiles of 16 rows, a row in
     a wave's registers."""

@@ -7,6 +7,7 @@ import torch
 from ..kernels import ops
 from .base import SplitStream, StepContext, settled
 from .linear import linear
+from .norms import as_tensor
 from .registry import register_block
 
 
@@ -91,12 +92,26 @@ class ParallelBlock:
     def forward(self, x: torch.Tensor, ctx: StepContext, cache, state, writes_cache: bool = True):
         if ctx.phases is not None:
             ctx.phases.mark(self.mixer_phase)
-        h = self.norm_mixer.forward(x, ctx, name="block_in")
+        # The norm is left pending where it can be: in steps of few rows the products that read it apply it to their own operand
+        # (one launch less), and a part that needs the rows themselves computes them once (`as_tensor`). A pending norm reads
+        # the stream when a product runs, so everything that reads h runs before anything adds into the stream: a feed-forward
+        # that can be run in two halves (`begin` / `finish`) makes its first product ahead of the mixer; any other gets the rows.
+        norm, ffn = self.norm_mixer, self.ffn
+        h = norm.lazy(x, ctx, name="block_in") if hasattr(norm, "lazy") else norm.forward(x, ctx, name="block_in")
+        begun = None
+        if ffn is not None:
+            if hasattr(ffn, "begin"):
+                begun = ffn.begin(h, ctx)
+            else:
+                h = as_tensor(h)
         self.mixer.forward(h, ctx, cache, state, x, writes_cache=writes_cache)
-        if self.ffn is not None:
+        if ffn is not None:
             if ctx.phases is not None:
                 ctx.phases.mark(self.ffn_phase)
-            self.ffn.forward(h, ctx, x)
+            if begun is not None:
+                ffn.finish(begun, ctx, x)
+            else:
+                ffn.forward(h, ctx, x)
         return None
 
 

@@ -71,22 +71,27 @@ class ClampedGLU:
         self.in_weight = store.fetch_joined([t["gate"], t["up"]], [(self.inner, self.width)] * 2, "matrix", "rows")
         self.down_weight = store.fetch(t["down"], (self.width, self.inner), "matrix")
 
-    def forward(self, h, ctx: StepContext, residual: Optional[torch.Tensor], out: Optional[torch.Tensor] = None):
-        """Adds the result into `residual` (float32 [n, width]), or leaves it in `out`."""
-        from ..kernels import ops
-        from .norms import as_tensor
-
-        h = as_tensor(h)
-        n = h.shape[0]
-        gu = ctx.workspace.get("glu_in", (n, 2 * self.inner), torch.float32)
+    def begin(self, h, ctx: StepContext) -> torch.Tensor:
+        """The first product, [gate | up] of h in 32 bits: everything of the feed-forward that reads its input. A block whose
+        sublayers read one pending norm of the stream runs this before any sublayer adds into the stream."""
+        gu = ctx.workspace.get("glu_in", (h.shape[0], 2 * self.inner), torch.float32)
         linear(h, self.in_weight, None, out=gu)
-        inner = ctx.workspace.get("ffn_inner", (n, self.inner), self.dtype)
+        return gu
+
+    def finish(self, gu: torch.Tensor, ctx: StepContext, residual: Optional[torch.Tensor], out: Optional[torch.Tensor] = None):
+        from ..kernels import ops
+
+        inner = ctx.workspace.get("ffn_inner", (gu.shape[0], self.inner), self.dtype)
         ops.glu_clamped(inner, gu, self.limit, self.slope, self.shift)
         if out is not None:
             linear(inner, self.down_weight, None, out=out)
         else:
             linear(inner, self.down_weight, None, residual=settled(residual))
         return None
+
+    def forward(self, h, ctx: StepContext, residual: Optional[torch.Tensor], out: Optional[torch.Tensor] = None):
+        """Adds the result into `residual` (float32 [n, width]), or leaves it in `out`."""
+        return self.finish(self.begin(h, ctx), ctx, residual, out=out)
 
 
 register_ffn("clamped_glu", ClampedGLU)

@@ -31,7 +31,7 @@ TILED_PARTS = True  # products of 33 to 64 rows that are added to the stream: ti
 
 
 def _fuses(a, w: torch.Tensor, residual) -> bool:
-    return (FOLD_NORM and isinstance(a, Normed) and getattr(a.norm, "fusable", None) == "layernorm" and residual is None
+    return (FOLD_NORM and isinstance(a, Normed) and getattr(a.norm, "fusable", None) in ("layernorm", "dyt") and residual is None
             and a.rows is None and a._tensor is None and w.dtype == torch.bfloat16 and a.x.dtype == torch.float32
             and a.x.is_contiguous() and a.n_rows <= FOLD_NORM_ROWS
             and ops.skinny_ln_pays(a.n_rows, w.shape[0], a.norm.width))
@@ -49,7 +49,10 @@ def linear(a, w: torch.Tensor, bias: Optional[torch.Tensor], *, out: Optional[to
         epilogue = ops.ACTIVATION_EPILOGUE[activation]
     if _fuses(a, w, residual):
         n = a.norm
-        ops.gemm_skinny_ln(a.x, n.weight, n.bias, n.eps, w, bias, out=out, epilogue=epilogue, kv=kv)
+        if n.fusable == "dyt":
+            ops.gemm_skinny_dyt(a.x, n.weight, n.bias, n.alpha, w, bias, out=out, epilogue=epilogue, kv=kv)
+        else:
+            ops.gemm_skinny_ln(a.x, n.weight, n.bias, n.eps, w, bias, out=out, epilogue=epilogue, kv=kv)
         return
     if isinstance(a, Normed):
         a = a.tensor()

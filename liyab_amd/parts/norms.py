@@ -118,6 +118,11 @@ class DynamicTanh:
 
     replayable = True
     takes_padding_rows = True
+    fusable = "dyt"  # the streaming product kernel knows how to fold this norm into its operand (steps of few rows)
+
+    def lazy(self, x: torch.Tensor, ctx: StepContext, rows: Optional[torch.Tensor] = None,
+             n_rows: Optional[int] = None, name: str = "normed") -> Normed:
+        return Normed(self, x, ctx, rows, n_rows, name)
 
     def __init__(self, spec, store, dtype: torch.dtype):
         self.width = spec.width

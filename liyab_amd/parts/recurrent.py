@@ -118,7 +118,6 @@ class StateSpace:
     def forward(self, h, ctx: StepContext, cache, state, residual: Optional[torch.Tensor], writes_cache: bool = True,
                 out: Optional[torch.Tensor] = None, proj: Optional[torch.Tensor] = None):
         """`proj`: the input projection's 32-bit rows, when the caller has made them (as columns of a wider product)."""
-        h = as_tensor(h)
         n, ws, inner, C = h.shape[0], ctx.workspace, self.inner, self.channels
         if proj is None:
             proj = ws.get("ssm_in", (n, self.in_weight.shape[0]), torch.float32)

@@ -132,7 +132,6 @@ class ScoredAttention:
                 writes_cache: bool = True, out: Optional[torch.Tensor] = None, proj: Optional[torch.Tensor] = None):
         """Adds the mixer's result into `residual`, or, with `out` (float32 [n, width]), leaves it there. `proj`: the input
         projection's 32-bit rows, when the caller has made them (as columns of a wider product)."""
-        h = as_tensor(h)
         n, ws, H, D, V = h.shape[0], ctx.workspace, self.n_head, self.head_dim, self.value_dim
         group = ctx.groups[cache.group]
         if proj is None:

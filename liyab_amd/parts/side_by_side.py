@@ -62,7 +62,6 @@ class SideBySide:
 
     def forward(self, h, ctx: StepContext, cache, state, residual: Optional[torch.Tensor], writes_cache: bool = True,
                 out: Optional[torch.Tensor] = None):
-        h = as_tensor(h)
         n, ws = h.shape[0], ctx.workspace
         a = ws.get("side_left", (n, self.width), torch.float32)
         b = ws.get("side_right", (n, self.width), torch.float32)
