@@ -260,6 +260,36 @@ def test_tanh_norm_alone(d, n):
     assert tt.rel_err(f64(out), plain.tanh_norm(f64(x)[[n - 1, 0]], t, "n")) < 1e-6
 
 
+@pytest.mark.parametrize("M,K,N", [(1, 96, 240), (1, 768, 2304), (8, 768, 2304), (3, 320, 512), (24, 1024, 64), (1, 64, 48), (2, 1600, 4800)])
+def test_the_norm_folded_into_a_product(M, K, N):
+    """The product that applies the norm to its own operand against the norm's kernel followed by the product."""
+    from liyab_amd.kernels import ops
+
+    rng = np.random.default_rng(11)
+    x, w, b = rand(rng, M, K, scale=2.0).to(DEV), rand(rng, K, scale=0.1, mean=1.0).to(DEV), rand(rng, K, scale=0.1).to(DEV)
+    alpha = torch.tensor([0.5], device=DEV)
+    W = rand(rng, N, K, scale=K ** -0.5).to(torch.bfloat16).to(DEV)
+    h = torch.empty(M, K, dtype=torch.bfloat16, device=DEV)
+    ops.dyt(h, x, w, b, alpha)
+    want = f64(h) @ f64(W).T
+    out = torch.full((M, N), float("nan"), dtype=torch.float32, device=DEV)
+    ops.gemm_skinny_dyt(x, w, b, alpha, W, None, out=out)
+    assert tt.rel_err(f64(out), want) < 1e-3  # (the two tanh differ by a rounding of the bfloat16 rows here and there)
+    exact = (np.tanh(0.5 * f64(x)) * f64(w) + f64(b)) @ f64(W).T
+    assert tt.rel_err(f64(out), exact) < 1e-2
+
+
+def test_the_recurrence_kernels_sizes():
+    """The sizes the host says the recurrence kernel takes are the ones its launcher takes."""
+    from liyab_amd.kernels import lib, ops
+
+    native = lib.load().liyab_scan_takes
+    for rows in (1, 3, 4, 8, 10, 16, 32, 64, 100, 128, 256, 300, 512, 600):
+        for cols in (1, 4, 8, 14, 16, 24, 48, 64, 100, 128, 256, 512, 600):
+            assert bool(native(rows, cols)) == ops.scan_takes(rows, cols), (rows, cols)
+    assert ops.scan_takes(64, 64) and ops.scan_takes(128, 128) and ops.scan_takes(128, 64) and not ops.scan_takes(64, 1000)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("width,ff,limit", [(64, 96, 1.5), (100, 50, 0.3), (72, 200, 50.0)])
 def test_clamped_feed_forward_alone(dtype, width, ff, limit):
