@@ -416,10 +416,10 @@ def mofulix_config(gpt2_cfg):
     mlp = {"kind": "dense", "ff": ff, "limit": 7.0}
     kinds = [
         {"type": "attention", "mixer": {"heads": H, "kv_heads": H, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "softcap": 30.0,
-                                        "rot": {"dims": hd, "base": 10000.0, "scaling": {"factor": 4.0, "low": 1.0, "high": 4.0, "original": 2048}}}},
+                                        "rot": {"dims": hd, "base": 10000.0, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}},
         {"type": "wkv", "mixer": {"heads": H, "dim": hd, "decay_rank": 64}},
         {"type": "parallel", "mixer": {"left": {"heads": H, "kv_heads": H, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "bias_max": 128, "bias_rows": 32,
-                                                "q_temp": {"coef": 0.1, "every": 256}},
+                                                "q_temp": {"coef": 0.1, "every": 512}},
                                        "right": {"heads": H, "vdim": hd, "state": 64, "groups": 1, "conv": 4, "norm_groups": 1}}},
     ]
     layers = [dict(json.loads(json.dumps(kinds[i % 3])), mlp=dict(mlp)) for i in range(L)]
