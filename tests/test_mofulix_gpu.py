@@ -683,6 +683,37 @@ def test_drawn_geometries_whole_and_mixed(seed, tmp_path):
         core.manager.check()
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_real_widths_in_long_steps(dtype, tmp_path):
+    """Heads of 64 and 128, a width of 512, prompts of hundreds of tokens in one step and in mixed batches: the tiles of the
+    large products, the matrix-core attention with capped and with biased scores (keys and values of one width and of two),
+    the recurrences with states of 64 x 64 and 128 x 64 a head."""
+    from liyab_amd.weights import write_random_model
+
+    par = {"left": biased(8, 4, 64, 64, 32, 100, q_temp=(0.2, 128)), "right": space(8, 64, 128, 2, 4, 1)}
+    cfg = config(1000, 512, 1e-5, 2.0, [
+        layer("attention", attention(8, 8, 64, softcap=25.0, rot=rot(64, 10000.0, (8.0, 1.0, 4.0, 256))), ff=1024, limit=6.0),
+        layer("wkv", wkv(8, 64, 32), ff=1024, limit=6.0),
+        layer("parallel", par, ff=1024, limit=6.0),
+        layer("attention", attention(4, 1, 128, rot=rot(32)), None),
+        layer("parallel", {"left": biased(4, 4, 128, 64, 16, 300), "right": space(4, 128, 16, 1, 2, 4)}, ff=768, limit=3.0),
+        layer("wkv", wkv(8, 64, 32), ff=1024, limit=6.0, weights_of=1),
+    ])
+    d = str(tmp_path / "m")
+    write_random_model(d, json.loads(json.dumps(cfg)), 31)
+    raw, tensors = read_model(d)
+    t = twin_tensors(tensors, dtype)
+    reqs = {f"r{i}": tt.random_tokens(900 + i, n, raw["vocab"]) for i, n in enumerate([330, 700, 45])}
+    ref = {rid: plain.forward(raw, t, toks) for rid, toks in reqs.items()}
+    steps = tt.schedule_whole(reqs)
+    core = make_core(d, dtype, tt.max_live_tokens(steps))
+    check_logits(tt.run_schedule(core, steps), reqs, ref, dtype, f"mofulix-wide whole {dtype}", family="mofulix-wide")
+    steps = tt.schedule_mixed(reqs, seed=3, max_live=3, portions=(2, 130, 64, 300, 17))
+    core = make_core(d, dtype, None, max_requests=3, num_pages=tt.max_live_pages(steps, 16))
+    check_logits(tt.run_schedule(core, steps), reqs, ref, dtype, f"mofulix-wide mixed {dtype}", family="mofulix-wide")
+    core.manager.check()
+
+
 def generate_greedy(raw, t, prompt, n_new):
     toks = list(prompt)
     for _ in range(n_new):
