@@ -362,8 +362,10 @@ token_shift_kernel(T* __restrict__ out, const T* __restrict__ h, const float* __
     const float* prev_state = state + static_cast<int64_t>(from_state ? slot : 0) * state_stride;
     for (int i = threadIdx.x; i < d; i += 256) {
         const float cur = to_float<T>(h[static_cast<int64_t>(t) * d + i]);
-        float prev = 0.0f;
-        if (p > 0) prev = from_step ? to_float<T>(h[static_cast<int64_t>(t - 1) * d + i]) : (from_state ? prev_state[i] : 0.0f);
+        // both candidates are asked for under no branch (a load under a branch is waited for where the branch ends)
+        const float before = to_float<T>(h[static_cast<int64_t>(max(t - 1, 0)) * d + i]);
+        const float kept = prev_state[i];
+        const float prev = p > 0 ? (from_step ? before : (from_state ? kept : 0.0f)) : 0.0f;
         const float diff = prev - cur;
         for (int c = 0; c < n_mix; ++c)
             out[(static_cast<int64_t>(t) * n_mix + c) * d + i] = from_float<T>(fmaf(diff, mu[c * d + i], cur));
