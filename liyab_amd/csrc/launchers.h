@@ -102,11 +102,13 @@ int liyab_scan_takes(int rows, int cols);
 int liyab_wkv_scan(void* out, int out_dtype, const float* r, const float* k, const float* v, const float* wraw, const float* gate, int64_t ld,
                    const float* w0, const float* u, const float* norm_w, float eps, float* state, int64_t state_stride, int n_slots,
                    const void* keep_src, int keep_dtype, int64_t keep_ld, int keep_width, int64_t keep_off, const int* seq_starts,
-                   const int* positions, const int* state_slots, int n_seqs, int H, int D, hipStream_t stream);
+                   const int* positions, const int* state_slots, int n_seqs, int H, int D, int seg_tokens, int max_segs, float* seg_state,
+                   float* seg_decay, hipStream_t stream);
 int liyab_ssd_scan(float* y, int64_t ldy, const float* xbc, int64_t ldx, const float* dtraw, int64_t ldp, const float* dt_bias,
                    const float* A_log, const float* Dskip, float* state, int64_t state_stride, int n_slots, const float* keep_src,
                    int64_t keep_ld, int keep_width, int keep_ring, int64_t keep_off, const int* seq_starts, const int* positions,
-                   const int* state_slots, int n_seqs, int H, int P, int N, int G, hipStream_t stream);
+                   const int* state_slots, int n_seqs, int H, int P, int N, int G, int seg_tokens, int max_segs, float* seg_state,
+                   float* seg_decay, hipStream_t stream);
 int liyab_token_shift(void* out, int dtype, const void* h, const float* mu, int n_mix, const float* state, int64_t state_stride, int n_slots,
                       const int* tok_seq, const int* positions, const int* seq_starts, const int* state_slots, int n, int d,
                       hipStream_t stream);

@@ -67,6 +67,10 @@ struct ScanArgs {
     const float *dt_bias, *A_log, *Dskip;
     int64_t ldy;
     int G, inner;
+    // long portions in segments (seg_tokens > 0): a workgroup a (segment, head) instead of a (request, head), in three passes
+    int n_seqs, seg_tokens, max_segs, phase;  // phase 0: the whole portion by one workgroup; 1: each segment from a zero state, for its end; 3: each segment from its true start
+    float* seg_state;       // [segments][H][rows][cols]: after pass 1 a segment's own end state, after the combining pass the state it starts from
+    float* seg_decay;       // [segments][H][rows]: the product of a segment's decays, a row
 };
 
 // PF: elements a thread fetches ahead of each staged array (0: none are fetched ahead; the staging loop takes any size).
@@ -76,7 +80,25 @@ template <int MODE, int REG, int PF, typename OutT>
 __global__ void __launch_bounds__(SCAN_THREADS)
 scan_kernel(ScanArgs a) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
-    const int s = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+    const int h = blockIdx.y, tid = threadIdx.x;
+    int s = blockIdx.x, seg_begin = -1, seg_end = -1;
+    bool last_seg = true;
+    if (a.seg_tokens > 0) {
+        // segment blockIdx.x in the order of the requests: which request's, and which of its segments (a workgroup past the last exits)
+        int g = blockIdx.x;
+        for (s = 0; s < a.n_seqs; ++s) {
+            const int b = a.seq_starts[s], len = a.seq_starts[s + 1] - b;
+            const int n_seg = (len + a.seg_tokens - 1) / a.seg_tokens;
+            if (g < n_seg) {
+                seg_begin = b + g * a.seg_tokens;
+                seg_end = min(seg_begin + a.seg_tokens, b + len);
+                last_seg = g == n_seg - 1;
+                break;
+            }
+            g -= n_seg;
+        }
+        if (seg_begin < 0 || (a.phase == 1 && last_seg)) return;  // (nobody needs the end state of a request's last segment from zero)
+    }
     const int R = a.rows, C = a.cols, CL = a.col_lanes;
     const int n_rb = SCAN_THREADS / CL;
     const int Rp = n_rb * a.rows_per;  // rows as staged: zeros behind the last (rows_per is a multiple of 4)
@@ -86,7 +108,7 @@ scan_kernel(ScanArgs a) {
     float* val = qr + SCAN_CHUNK * Rp;            // [CHUNK][CL]
     float* part = val + SCAN_CHUNK * CL;          // [CHUNK][n_rb][CL]
 
-    const int begin = a.seq_starts[s], end = a.seq_starts[s + 1];
+    const int begin = seg_begin >= 0 ? seg_begin : a.seq_starts[s], end = seg_begin >= 0 ? seg_end : a.seq_starts[s + 1];
     const int slot = a.state_slots[s];
     const bool slot_ok = slot >= 0 && slot < a.n_slots;
     const int cl_shift = __builtin_ctz(CL);  // (CL is a power of two)
@@ -94,12 +116,16 @@ scan_kernel(ScanArgs a) {
     const int i0 = rb * a.rows_per;
     float* S_glob = a.state + static_cast<int64_t>(slot_ok ? slot : 0) * a.state_stride + static_cast<int64_t>(h) * R * C;
     const bool fresh = a.positions[begin] == 0;
+    float* S_seg = a.seg_state + (static_cast<int64_t>(blockIdx.x) * a.H + h) * R * C;  // (read or written in passes 1 and 3 only)
 
-    float S[REG], bonus[MODE == 0 ? REG : 1];
+    float S[REG], bonus[MODE == 0 ? REG : 1], prod[REG];
 #pragma unroll
     for (int ii = 0; ii < REG; ++ii) {
         const int i = i0 + ii;
-        S[ii] = (ii < a.rows_per && i < R && j < C && slot_ok && !fresh) ? S_glob[static_cast<int64_t>(i) * C + j] : 0.0f;
+        const bool mine = ii < a.rows_per && i < R && j < C;
+        prod[ii] = 1.0f;
+        if (a.phase == 0) S[ii] = (mine && slot_ok && !fresh) ? S_glob[static_cast<int64_t>(i) * C + j] : 0.0f;
+        else S[ii] = (mine && a.phase == 3) ? S_seg[static_cast<int64_t>(i) * C + j] : 0.0f;
         if (MODE == 0) bonus[ii] = (ii < a.rows_per && i < R) ? a.u[h * R + i] : 0.0f;
     }
     const int g = MODE == 1 ? h / (a.H / a.G) : 0;
@@ -216,40 +242,49 @@ scan_kernel(ScanArgs a) {
             }
         };
         operands(0);
-        for (int tt = 0; tt < len; ++tt) {
-            float4 cd[REG / 4], ck[REG / 4], cq[REG / 4];
-            const float vj = nv;
+        auto tokens = [&](auto first_pass) {
+            constexpr bool kEndOnly = decltype(first_pass)::value;  // pass 1: the state and the decays' product, no outputs
+            for (int tt = 0; tt < len; ++tt) {
+                float4 cd[REG / 4], ck[REG / 4], cq[REG / 4];
+                const float vj = nv;
 #pragma unroll
-            for (int i4 = 0; i4 < REG / 4; ++i4) {
-                cd[i4] = nd[i4];
-                ck[i4] = nk[i4];
-                cq[i4] = nq[i4];
-            }
-            operands(min(tt + 1, len - 1));
-            float acc0 = 0.0f, acc1 = 0.0f;
+                for (int i4 = 0; i4 < REG / 4; ++i4) {
+                    cd[i4] = nd[i4];
+                    ck[i4] = nk[i4];
+                    cq[i4] = nq[i4];
+                }
+                operands(min(tt + 1, len - 1));
+                float acc0 = 0.0f, acc1 = 0.0f;
 #pragma unroll
-            for (int i4 = 0; i4 < REG / 4; ++i4) {
-                if (4 * i4 < a.rows_per) {
-                    const float dd[4] = {cd[i4].x, cd[i4].y, cd[i4].z, cd[i4].w}, kk[4] = {ck[i4].x, ck[i4].y, ck[i4].z, ck[i4].w},
-                                qv[4] = {cq[i4].x, cq[i4].y, cq[i4].z, cq[i4].w};
+                for (int i4 = 0; i4 < REG / 4; ++i4) {
+                    if (4 * i4 < a.rows_per) {
+                        const float dd[4] = {cd[i4].x, cd[i4].y, cd[i4].z, cd[i4].w}, kk[4] = {ck[i4].x, ck[i4].y, ck[i4].z, ck[i4].w},
+                                    qv[4] = {cq[i4].x, cq[i4].y, cq[i4].z, cq[i4].w};
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const int ii = 4 * i4 + e;
-                        const float kin = kk[e] * vj;
-                        float& acc = e % 2 ? acc1 : acc0;
-                        if (MODE == 0) {
-                            acc = fmaf(qv[e], fmaf(bonus[ii], kin, S[ii]), acc);
-                            S[ii] = fmaf(dd[e], S[ii], kin);
-                        } else {
-                            S[ii] = fmaf(dd[e], S[ii], kin);
-                            acc = fmaf(qv[e], S[ii], acc);
+                        for (int e = 0; e < 4; ++e) {
+                            const int ii = 4 * i4 + e;
+                            const float kin = kk[e] * vj;
+                            float& acc = e % 2 ? acc1 : acc0;
+                            if constexpr (kEndOnly) {
+                                S[ii] = fmaf(dd[e], S[ii], kin);
+                                prod[ii] *= dd[e];
+                            } else if (MODE == 0) {
+                                acc = fmaf(qv[e], fmaf(bonus[ii], kin, S[ii]), acc);
+                                S[ii] = fmaf(dd[e], S[ii], kin);
+                            } else {
+                                S[ii] = fmaf(dd[e], S[ii], kin);
+                                acc = fmaf(qv[e], S[ii], acc);
+                            }
                         }
                     }
                 }
+                if constexpr (!kEndOnly) part[(tt * n_rb + rb) * CL + j] = acc0 + acc1;
             }
-            part[(tt * n_rb + rb) * CL + j] = acc0 + acc1;
-        }
+        };
+        if (a.phase == 1) tokens(std::true_type{});
+        else tokens(std::false_type{});
         __syncthreads();
+        if (a.phase == 1) continue;  // (no outputs in pass 1)
         if (MODE == 0) {
             // a wave a token: the head's outputs, their root mean square, the weight and the gate
             const int wave = tid / kWave, lane = tid % kWave;
@@ -280,7 +315,18 @@ scan_kernel(ScanArgs a) {
             }
         }
     }
-    if (slot_ok) {
+    if (a.phase == 1) {
+        // the segment's end state from zero and the product of its decays, for the pass that strings the segments together
+        float* P_seg = a.seg_decay + (static_cast<int64_t>(blockIdx.x) * a.H + h) * R;
+#pragma unroll
+        for (int ii = 0; ii < REG; ++ii) {
+            const int i = i0 + ii;
+            if (ii < a.rows_per && i < R && j < C) S_seg[static_cast<int64_t>(i) * C + j] = S[ii];
+            if (ii < a.rows_per && i < R && j == 0) P_seg[i] = prod[ii];
+        }
+        return;
+    }
+    if (slot_ok && last_seg) {
 #pragma unroll
         for (int ii = 0; ii < REG; ++ii) {
             const int i = i0 + ii;
@@ -288,7 +334,7 @@ scan_kernel(ScanArgs a) {
         }
         if (h == 0 && a.keep_src != nullptr && a.keep_ring > 0) {
             float* dst = a.state + static_cast<int64_t>(slot) * a.state_stride + a.keep_off;
-            const int first = max(begin, end - a.keep_ring);
+            const int first = max(a.seq_starts[s], end - a.keep_ring);  // (of the request's rows, not of its last segment's only)
             for (int t = first; t < end; ++t) {
                 const int place = a.positions[t] % a.keep_ring;
                 for (int c = tid; c < a.keep_width; c += SCAN_THREADS) {
@@ -296,6 +342,45 @@ scan_kernel(ScanArgs a) {
                     dst[static_cast<int64_t>(place) * a.keep_width + c] =
                         a.keep_bf16 ? bf16_to_float(static_cast<const bf16_t*>(a.keep_src)[at]) : static_cast<const float*>(a.keep_src)[at];
                 }
+            }
+        }
+    }
+}
+
+// Between the two passes over a long portion's segments: the state each segment starts from. A workgroup a (request, head)
+// walks the request's segments in order, S <- decays' product * S + the segment's own end state, and leaves in seg_state what
+// each segment starts from (the first: the slot's state, or zeros at position 0).
+__global__ void __launch_bounds__(256)
+scan_combine_kernel(ScanArgs a) {
+    const int s = blockIdx.x, h = blockIdx.y;
+    int g0 = 0;
+    for (int q = 0; q < s; ++q) g0 += (a.seq_starts[q + 1] - a.seq_starts[q] + a.seg_tokens - 1) / a.seg_tokens;
+    const int begin = a.seq_starts[s];
+    const int n_seg = (a.seq_starts[s + 1] - begin + a.seg_tokens - 1) / a.seg_tokens;
+    const int slot = a.state_slots[s];
+    const bool from_slot = slot >= 0 && slot < a.n_slots && a.positions[begin] != 0;
+    const int R = a.rows, C = a.cols;
+    const int e = blockIdx.z * 256 + threadIdx.x;  // an element of the state a thread
+    if (e >= R * C) return;
+    const int i = e / C;
+    const float* S0 = a.state + static_cast<int64_t>(from_slot ? slot : 0) * a.state_stride + static_cast<int64_t>(h) * R * C;
+    float S = from_slot ? S0[e] : 0.0f;
+    // eight segments' values are asked for together, ahead of the chain that uses them (a load behind a store to the same
+    // array is not moved ahead of it by the compiler)
+    constexpr int kBatch = 8;
+    for (int c0 = 0; c0 < n_seg; c0 += kBatch) {
+        float own[kBatch], dec[kBatch];
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+            const int64_t g = g0 + min(c0 + u, n_seg - 1);
+            own[u] = a.seg_state[(g * a.H + h) * R * C + e];  // (a request's last segment has none: read and dropped)
+            dec[u] = a.seg_decay[(g * a.H + h) * R + i];
+        }
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+            if (c0 + u < n_seg) {
+                a.seg_state[(static_cast<int64_t>(g0 + c0 + u) * a.H + h) * R * C + e] = S;
+                if (c0 + u + 1 < n_seg) S = fmaf(dec[u], S, own[u]);
             }
         }
     }
@@ -328,6 +413,16 @@ static void launch_scan_one(const ScanArgs& a, int n_seqs, size_t smem, hipStrea
     if (smem > 48 * 1024) {
         static bool allowed = false;  // (once a kernel: more dynamic LDS than the default limit)
         if (!allowed) allowed = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(SCAN_MAX_LDS)) == hipSuccess;
+    }
+    if (a.seg_tokens > 0) {
+        // segments side by side: each from a zero state for its end, the ends strung together, each again from its true start
+        ScanArgs p = a;
+        p.phase = 1;
+        kern<<<dim3(a.max_segs, a.H), SCAN_THREADS, smem, stream>>>(p);
+        scan_combine_kernel<<<dim3(n_seqs, a.H, (a.rows * a.cols + 255) / 256), 256, 0, stream>>>(p);
+        p.phase = 3;
+        kern<<<dim3(a.max_segs, a.H), SCAN_THREADS, smem, stream>>>(p);
+        return;
     }
     kern<<<dim3(n_seqs, a.H), SCAN_THREADS, smem, stream>>>(a);
 }
@@ -439,7 +534,7 @@ extern "C" int liyab_wkv_scan(void* out, int out_dtype, const float* r, const fl
                               int64_t ld, const float* w0, const float* u, const float* norm_w, float eps, float* state, int64_t state_stride,
                               int n_slots, const void* keep_src, int keep_dtype, int64_t keep_ld, int keep_width, int64_t keep_off,
                               const int* seq_starts, const int* positions, const int* state_slots, int n_seqs, int H, int D,
-                              hipStream_t stream) {
+                              int seg_tokens, int max_segs, float* seg_state, float* seg_decay, hipStream_t stream) {
     LIYAB_REQUIRE(out && r && k && v && wraw && gate && w0 && u && norm_w && state && seq_starts && positions && state_slots, "wkv_scan: null pointer");
     LIYAB_REQUIRE(n_seqs >= 0 && H > 0 && D > 0 && n_slots > 0, "wkv_scan: bad sizes");
     LIYAB_REQUIRE(ld >= static_cast<int64_t>(H) * D, "wkv_scan: rows shorter than heads x head size");
@@ -451,6 +546,8 @@ extern "C" int liyab_wkv_scan(void* out, int out_dtype, const float* r, const fl
     int reg, pf;
     LIYAB_REQUIRE(scan_shape(D, D, &a.col_lanes, &a.rows_per, &reg, &pf, &smem), "wkv_scan: heads of %d are not taken", D);
     if (n_seqs == 0) return 0;
+    LIYAB_REQUIRE(seg_tokens >= 0 && (seg_tokens == 0 || (max_segs > 0 && seg_state && seg_decay)), "scan: segments need their count and scratch");
+    a.n_seqs = n_seqs; a.seg_tokens = seg_tokens; a.max_segs = max_segs; a.seg_state = seg_state; a.seg_decay = seg_decay;
     a.state = state; a.state_stride = state_stride; a.n_slots = n_slots;
     a.seq_starts = seq_starts; a.positions = positions; a.state_slots = state_slots;
     a.H = H; a.rows = D; a.cols = D;
@@ -465,7 +562,8 @@ extern "C" int liyab_wkv_scan(void* out, int out_dtype, const float* r, const fl
 extern "C" int liyab_ssd_scan(float* y, int64_t ldy, const float* xbc, int64_t ldx, const float* dtraw, int64_t ldp, const float* dt_bias,
                               const float* A_log, const float* Dskip, float* state, int64_t state_stride, int n_slots, const float* keep_src,
                               int64_t keep_ld, int keep_width, int keep_ring, int64_t keep_off, const int* seq_starts, const int* positions,
-                              const int* state_slots, int n_seqs, int H, int P, int N, int G, hipStream_t stream) {
+                              const int* state_slots, int n_seqs, int H, int P, int N, int G, int seg_tokens, int max_segs, float* seg_state,
+                              float* seg_decay, hipStream_t stream) {
     LIYAB_REQUIRE(y && xbc && dtraw && dt_bias && A_log && Dskip && state && seq_starts && positions && state_slots, "ssd_scan: null pointer");
     LIYAB_REQUIRE(n_seqs >= 0 && H > 0 && P > 0 && N > 0 && G > 0 && H % G == 0 && n_slots > 0, "ssd_scan: bad sizes");
     const int64_t inner = static_cast<int64_t>(H) * P;
@@ -477,6 +575,8 @@ extern "C" int liyab_ssd_scan(float* y, int64_t ldy, const float* xbc, int64_t l
     int reg, pf;
     LIYAB_REQUIRE(scan_shape(N, P, &a.col_lanes, &a.rows_per, &reg, &pf, &smem), "ssd_scan: a state of %d x %d a head is not taken", N, P);
     if (n_seqs == 0) return 0;
+    LIYAB_REQUIRE(seg_tokens >= 0 && (seg_tokens == 0 || (max_segs > 0 && seg_state && seg_decay)), "scan: segments need their count and scratch");
+    a.n_seqs = n_seqs; a.seg_tokens = seg_tokens; a.max_segs = max_segs; a.seg_state = seg_state; a.seg_decay = seg_decay;
     a.state = state; a.state_stride = state_stride; a.n_slots = n_slots;
     a.seq_starts = seq_starts; a.positions = positions; a.state_slots = state_slots;
     a.H = H; a.rows = N; a.cols = P;

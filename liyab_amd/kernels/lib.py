@@ -93,9 +93,9 @@ _SIGNATURES = {
     "liyab_activate": [P, c_int, c_int64, P, c_int64, c_int, c_int, c_int, P],
     "liyab_mean_norm_add": [P, P, P, P, P, c_float, c_float, c_int, c_int, P],
     "liyab_wkv_scan": [P, c_int, P, P, P, P, P, c_int64, P, P, P, c_float, P, c_int64, c_int, P, c_int, c_int64, c_int, c_int64, P, P, P,
-                       c_int, c_int, c_int, P],
+                       c_int, c_int, c_int, c_int, c_int, P, P, P],
     "liyab_ssd_scan": [P, c_int64, P, c_int64, P, c_int64, P, P, P, P, c_int64, c_int, P, c_int64, c_int, c_int, c_int64, P, P, P, c_int,
-                       c_int, c_int, c_int, c_int, P],
+                       c_int, c_int, c_int, c_int, c_int, c_int, P, P, P],
     "liyab_token_shift": [P, c_int, P, P, c_int, P, c_int64, c_int, P, P, P, P, c_int, c_int, P],
     "liyab_conv_act": [P, c_int64, P, c_int64, P, P, c_int, P, c_int64, c_int, P, P, P, P, c_int, c_int, P],
     "liyab_gated_group_norm": [P, c_int, P, c_int64, P, c_int64, P, c_float, c_int, c_int, c_int, P],

@@ -1359,6 +1359,22 @@ def scan_takes(rows: int, cols: int) -> bool:
     return per <= 64 and 4 * (3 * 16 * staged + 2 * 16 * lanes + 16 * threads) <= 128 * 1024
 
 
+SCAN_SEGMENT = 64  # tokens a segment where a long portion's recurrence runs in segments side by side
+SCAN_SEGMENT_FROM = 192  # the longest portion of a step from which it does
+
+
+def _scan_segments(ctx, n: int, n_head: int, rows: int, cols: int):
+    """(tokens a segment, the most segments, scratch for the segments' states, for their decays) for a step's recurrence: in
+    segments side by side when some request brings a long portion, else (0, 0, None, None). The grids follow from the step's
+    rows and requests, never from the portions' lengths."""
+    if ctx.host.max_q_len < SCAN_SEGMENT_FROM:
+        return 0, 0, None, None
+    most = -(-n // SCAN_SEGMENT) + ctx.n_seqs
+    state = ctx.workspace.get("scan_seg_state", (most, n_head, rows, cols), torch.float32)
+    decay = ctx.workspace.get("scan_seg_decay", (most, n_head, rows), torch.float32)
+    return SCAN_SEGMENT, most, state.data_ptr(), decay.data_ptr()
+
+
 def _step_lists(ctx, n: int) -> None:
     _i32(ctx.tok_seq, "tok_seq", n)
     _i32(ctx.positions, "positions", n)
@@ -1416,7 +1432,7 @@ def wkv_scan(out: torch.Tensor, proj: torch.Tensor, w0: torch.Tensor, u: torch.T
     _lib.call("liyab_wkv_scan", out.data_ptr(), dtype_code(out.dtype), p, p + 4 * HD, p + 8 * HD, p + 16 * HD, p + 12 * HD, ld, w0.data_ptr(),
               u.data_ptr(), norm_w.data_ptr(), float(eps), state.data_ptr(), stride, state.shape[0], h.data_ptr(), dtype_code(h.dtype),
               h.shape[1], h.shape[1], H * D * D, ctx.seq_starts.data_ptr(), ctx.positions.data_ptr(), ctx.state_slots.data_ptr(), ctx.n_seqs,
-              H, D, _stream())
+              H, D, *_scan_segments(ctx, n, H, D, D), _stream())
 
 
 def conv_act(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], state: Optional[torch.Tensor],
@@ -1476,7 +1492,8 @@ def ssd_scan(y: torch.Tensor, xbc: torch.Tensor, dt_raw: torch.Tensor, dt_bias: 
     _step_lists(ctx, n)
     _lib.call("liyab_ssd_scan", y.data_ptr(), ldy, xbc.data_ptr(), ldx, dt_raw.data_ptr(), ldp, dt_bias.data_ptr(), a_log.data_ptr(),
               d_skip.data_ptr(), state.data_ptr(), stride, state.shape[0], kptr, kld, kw, keep_ring if kptr is not None else 0, inner * N,
-              ctx.seq_starts.data_ptr(), ctx.positions.data_ptr(), ctx.state_slots.data_ptr(), ctx.n_seqs, H, P, N, G, _stream())
+              ctx.seq_starts.data_ptr(), ctx.positions.data_ptr(), ctx.state_slots.data_ptr(), ctx.n_seqs, H, P, N, G,
+              *_scan_segments(ctx, n, H, N, P), _stream())
 
 
 def gated_group_norm(out: torch.Tensor, y: torch.Tensor, z: torch.Tensor, weight: torch.Tensor, eps: float, groups: int) -> None:

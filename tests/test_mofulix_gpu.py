@@ -240,6 +240,9 @@ def _inputs(p, rng, n, scale=1.0):
 
 MIXER_TOL = {"float32": 2e-5, "bfloat16": 3e-2}
 PORTIONS = ((75,), (25, 1, 9, 1, 1, 2, 36), (2,) * 10 + (1,) * 5 + (50,), (1,) * 75)
+# portions long enough to run in segments side by side: a whole number of segments, one token more, one less, and a long
+# portion that starts from a state earlier portions left
+LONG_PORTIONS = ((257,), (192, 1, 64), (3, 255), (320,))
 
 
 @pytest.mark.parametrize("d,n", [(96, 5), (100, 33), (2500, 3)])
@@ -313,7 +316,8 @@ def test_wkv_alone_in_portions(dtype, m):
     slot that was used before starts from zeros whatever the slot holds."""
     p = _Layer(dtype, layer("wkv", m), width=72)
     rng = np.random.default_rng(3)
-    for k, portions in enumerate(PORTIONS):
+    # (a decay of rank 1 is one bfloat16 number a token: over hundreds of tokens its rounding alone passes the tolerance)
+    for k, portions in enumerate(PORTIONS + (LONG_PORTIONS if dtype == "float32" or m["decay_rank"] > 1 else ())):
         x, xs = _inputs(p, rng, sum(portions))
         want = plain.wkv(xs, p.t, "l0.mix.", m, p.eps)
         got = _mixer_alone(p, x, portions, rid=f"w{k}")
@@ -348,7 +352,7 @@ def test_state_space_alone_in_portions(dtype, m):
     p = _Layer(dtype, entry, width=72)
     rng = np.random.default_rng(5)
     core, mix = p.core, p.block.mixer.right
-    for k, portions in enumerate(PORTIONS):
+    for k, portions in enumerate(PORTIONS + LONG_PORTIONS):
         x, xs = _inputs(p, rng, sum(portions))
         want = plain.state_space(xs, p.t, "l0.mix.right.", m, p.eps)
         rid = f"s{k}"
