@@ -16,6 +16,10 @@
 // the request's last input rows for the next step (the previous token's input of a token shift, the last
 // taps - 1 inputs of a short convolution), at ring place position % ring: after every read of them, since
 // the kernels that read them ran before this one.
+// A step with a long portion runs the same kernel over segments of the portions side by side (seg_tokens > 0), in three
+// launches: every segment from a zero state for its end state and the product of its decays; scan_combine_kernel, which
+// strings a request's segments together and leaves each the state it starts from; every segment again from that state,
+// with outputs. Decays are only ever multiplied, and the grids follow from the step's rows and requests alone.
 //
 // liyab_token_shift: m_c[t] = h[t] + (h[t - 1] - h[t]) * mu_c for each of n_mix learned mixes (a token's mixes side by side
 //   in its row of the output, [n, n_mix * d]), the previous
